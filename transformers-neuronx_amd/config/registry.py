@@ -40,7 +40,7 @@ _ARCHITECTURES: Dict[str, Architecture] = {}
 # its import before a model folder is read). A program that is started apart (a command line) learns of
 # packages from outside through the environment: TNX_ARCHITECTURE_PACKAGES holds module names, separated
 # by commas, that are importable from where it runs.
-ARCHITECTURE_PACKAGES: List[str] = ["transformers_neuronx_amd.opt"]
+ARCHITECTURE_PACKAGES: List[str] = ["transformers_neuronx_amd.opt", "transformers_neuronx_amd.ratesun"]
 PACKAGES_VARIABLE = "TNX_ARCHITECTURE_PACKAGES"
 
 
@@ -74,7 +74,9 @@ def _load_builtin():
 def resolve(raw: Dict[str, Any]) -> Architecture:
     """The architecture a config.json names."""
     _load_builtin()
-    names = raw.get("architectures") or []
+    names = list(raw.get("architectures") or [])
+    if isinstance(raw.get("architecture"), str):       # a config.json that names its one architecture so
+        names.append(raw["architecture"])
     for n in names:
         if n in _ARCHITECTURES:
             return _ARCHITECTURES[n]

@@ -74,6 +74,13 @@ class StepContext:
     cached_lens_host: np.ndarray = None
     slots_host: np.ndarray = None
     plans: Dict = field(default_factory=dict)    # launch plans the kernel backend keeps per step
+    # What several parts of one pass through the model share (a table's rows looked up once a step for all
+    # layers): emptied by the model at the start of every pass.
+    memo: Dict = field(default_factory=dict)
+    # The per-request state of parts that are no mixers (`Part.state_need`), as `LayerCache`s: the embedding's,
+    # and that of the call of the run order under way (set by the model before each block runs).
+    input_state: Optional[object] = None
+    call_state: Optional[object] = None
 
     @property
     def max_run(self) -> int:

@@ -29,7 +29,8 @@ class _Layer:
         s = self.spec
         return [(self.mixer, s.prefix + s.mixer_name), (self.feed_forward, s.prefix + s.feed_forward_name),
                 (self.mixer_norm, s.prefix + s.mixer_norm_name),
-                (self.feed_forward_norm, s.prefix + s.feed_forward_norm_name)]
+                (self.feed_forward_norm, s.prefix + s.feed_forward_norm_name),
+                (self.block, s.prefix)]          # what the arrangement itself reads
 
     def param_decls(self) -> List[ParamDecl]:
         return [d for part, prefix in self._named() for d in part.param_decls(prefix)]
@@ -59,6 +60,22 @@ class DecoderModel:
                 written.add(cid)
             elif cid not in written:
                 raise ValueError(f"layer {layer} reads cache {cid} before the call that writes it")
+        # parts other than mixers that keep something per request get a cache of their own, numbered after
+        # the run order's: the embedding, and every call's block (a layer named twice keeps two)
+        nxt = max((cid for _, cid, _ in self.schedule), default=-1) + 1
+        self.part_state_needs: Dict[int, CacheNeed] = {}
+        self.input_state_id = None
+        if self.embedding.state_need() is not None:
+            self.input_state_id = nxt
+            self.part_state_needs[nxt] = self.embedding.state_need()
+            nxt += 1
+        self.call_state_ids: List[Optional[int]] = []
+        for layer, _, _ in self.schedule:
+            need = self.layers[layer].block.state_need()
+            self.call_state_ids.append(nxt if need is not None else None)
+            if need is not None:
+                self.part_state_needs[nxt] = need
+                nxt += 1
         self.loaded = False
         parts = [self.embedding, self.embedding.position, self.head] + ([self.head.norm] if self.head.norm else [])
         for l in self.layers:
@@ -78,8 +95,10 @@ class DecoderModel:
         return decls
 
     def cache_needs(self) -> Dict[int, Optional[CacheNeed]]:
-        """{cache id: need} of the calls that write a cache."""
-        return {cid: self.layers[layer].mixer.cache_need() for layer, cid, writes in self.schedule if writes}
+        """{cache id: need} of the calls that write a cache, and of the parts that keep state of their own."""
+        needs = {cid: self.layers[layer].mixer.cache_need() for layer, cid, writes in self.schedule if writes}
+        needs.update(self.part_state_needs)
+        return needs
 
     def step_planners(self) -> Dict[str, object]:
         """The step planners that the parts bring with them."""
@@ -105,7 +124,8 @@ class DecoderModel:
         per_token = self.embedding.flops_per_token(keys)
         for layer, _, _ in self.schedule:
             l = self.layers[layer]
-            per_token += sum(p.flops_per_token(keys) for p in (l.mixer, l.feed_forward, l.mixer_norm, l.feed_forward_norm))
+            per_token += sum(p.flops_per_token(keys) for p in (l.mixer, l.feed_forward, l.mixer_norm, l.feed_forward_norm,
+                                                               l.block))
         return tokens * per_token + wanted * self.head.flops_per_token(keys)
 
     def cache_bytes_read(self, keys: float, dtype: torch.dtype, page_size: int = 1) -> float:
@@ -128,7 +148,8 @@ class DecoderModel:
              finish: bool = True) -> "DecoderModel":
         """`finish=False` leaves out what the blocks do once their parts have their tensors (`finish_load`
         does it later: the caller has something to do to the weights in between)."""
-        tensors = load_tensors(self.param_decls(), source, dtype, device, self.spec.base_model_prefix, cast_float32)
+        tensors = load_tensors(self.param_decls(), source, dtype, device, self.spec.base_model_prefix, cast_float32,
+                               self.spec.unread)
         self.embedding.load(tensors, "", ops, dtype)
         for layer in self.layers:
             layer.load(tensors, ops, dtype, finish)
@@ -148,10 +169,14 @@ class DecoderModel:
         """Logits float32 `[len(ctx.logits_rows), vocab]` for the step `ctx` describes."""
         first_block = self.layers[self.schedule[0][0]].block if self.schedule else None
         want_compute = bool(getattr(first_block, "reads_compute_copy", False))
+        ctx.memo = {}
+        ctx.input_state = caches[self.input_state_id] if self.input_state_id is not None else None
         stream: Stream = self.embedding.forward(ctx, want_compute)
         debug.tap("embedding", stream.x)
         for call, (layer, cid, writes) in enumerate(self.schedule):
             cache = caches[cid] if writes else caches[cid].reader()
+            state_id = self.call_state_ids[call]
+            ctx.call_state = caches[state_id] if state_id is not None else None
             stream = self.layers[layer].block.forward(stream, ctx, cache)
             debug.tap(f"call{call}.layer{layer}", stream.x)
         return debug.tap("logits", self.head.forward(stream, ctx))

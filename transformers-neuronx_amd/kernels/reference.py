@@ -185,6 +185,156 @@ class ReferenceOps:
             out[s:e] = o.permute(1, 0, 2).reshape(e - s, num_heads * head_size)
         return out.to(self.dtype)
 
+
+    # ---------------------------------------------------------------- parts of other designs
+
+    def _resolved(self, token_ids, kept_tokens):
+        ids = token_ids.long()
+        if kept_tokens is not None:
+            ids = torch.where(ids < 0, kept_tokens.long()[(-1 - ids).clamp(min=0)], ids)
+        return ids
+
+    def embed_pairs(self, token_ids, table, pairs, buckets, mul_prev, mul_cur, ctx, last_token, kept_tokens=None):
+        """float32 `table[token] + pairs[row]`, row = (previous * mul_prev + token * mul_cur) mod buckets, and
+        `buckets` at position 0; the token before a step's first of a request is `last_token[slot, 0]`, which
+        then takes the request's last token of this step."""
+        ids = self._resolved(token_ids, kept_tokens)
+        starts = ctx.run_start.long()
+        first = torch.zeros_like(ids, dtype=torch.bool)
+        first[starts[:-1]] = True
+        slots = ctx.slots.long()
+        before = torch.roll(ids, 1)
+        before[starts[:-1]] = last_token[slots, 0].long()
+        rows = (before * mul_prev + ids * mul_cur) % buckets
+        rows = torch.where(ctx.positions.long() == 0, torch.full_like(rows, buckets), rows)
+        last_token[slots, 0] = ids[starts[1:] - 1].to(last_token.dtype)
+        return table[ids].float() + pairs[rows].float()
+
+    def norm_add(self, y, weight, bias, eps, center, residual, mult=1.0, out=None):
+        """float32 `residual + mult * norm(y)`; `center` as in `layernorm`."""
+        normed = self.layernorm(y, weight, bias, eps, torch.float32, True, False, center)[0]
+        result = residual.float() + mult * normed
+        if out is not None:
+            out.copy_(result)
+            return out
+        return result
+
+    def input_conv(self, h, weight, state, which, ctx, dtype):
+        """`h + conv(h)`: conv(h)_t = sum_j weight[:, j] h_(t - taps + 1 + j) over the tokens of t's own request;
+        the taps - 1 inputs before a step's first token of a request come from `state[slot, which]`
+        (`[taps - 1, width]`, oldest first, zeros at a request's start), which then takes the last ones."""
+        taps = weight.shape[1]
+        out = torch.empty_like(h)
+        start = 0
+        for r in range(ctx.num_requests):
+            n, slot = int(ctx.run_lens_host[r]), int(ctx.slots_host[r])
+            run = h[start:start + n].float()
+            if taps > 1:
+                seq = torch.cat([state[slot, which].float(), run], dim=0)
+                state[slot, which] = seq[-(taps - 1):]
+            else:
+                seq = run
+            acc = run.clone()
+            for j in range(taps):
+                acc = acc + weight[:, j].float()[None, :] * seq[j:j + n]
+            out[start:start + n] = acc
+            start += n
+        return out.to(dtype)
+
+    def poly_norm(self, z, coeffs, eps):
+        """a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over a row; float32 in, compute
+        dtype out."""
+        z = z.float()
+        c = coeffs.float()
+
+        def unit(v):
+            return v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps)
+        return (c[0] * unit(z) + c[1] * unit(z * z) + c[2] * unit(z * z * z) + c[3]).to(self.dtype)
+
+    def mul_columns(self, g, rows, offset):
+        """`g * rows[:, offset:offset + g.shape[1]]`, rounded once."""
+        return (g.float() * rows[:, offset:offset + g.shape[1]].float()).to(self.dtype)
+
+    def weighted_sum(self, history, weights, count):
+        """float32 `sum_j weights[j] history[j]` over the first `count` slots of `history` `[slots, T, width]`."""
+        out = torch.zeros_like(history[0])
+        for j in range(count):
+            out = out + weights[j] * history[j]
+        return out
+
+    @staticmethod
+    def _turn(x, positions, freqs):
+        """Pairs (2i, 2i + 1) of the last axis of `x` `[T, ..., r]` turned by positions * freqs[i]; float32."""
+        dims = 2 * freqs.numel()
+        angle = positions.float().reshape([-1] + [1] * (x.dim() - 1)) * freqs.float()
+        cos, sin = torch.cos(angle), torch.sin(angle)
+        u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+        out = x.clone()
+        out[..., 0:dims:2] = u * cos - v * sin
+        out[..., 1:dims:2] = v * cos + u * sin
+        return out
+
+    def latent_norms(self, down, q_rank, kv_rank, rot, q_weight, kv_weight, eps, freqs, ctx, view, latent_pages,
+                     rotated_pages):
+        """`down` float32 `[T, q_rank + kv_rank + rot]`: the first q_rank elements, scaled to unit root mean
+        square and weighted, come back in the compute dtype; the next kv_rank likewise go to the tokens' places
+        in `latent_pages`, the last `rot`, turned by the position, to `rotated_pages` (kv_rank 0: none)."""
+        x = down.float()
+
+        def rms(v, w):
+            return v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps) * w.float()
+        c_q = rms(x[:, :q_rank], q_weight).to(self.dtype)
+        if kv_rank:
+            pos = ctx.positions.long()
+            page = view.block_table[ctx.token_request.long(), pos // view.page_size].long()
+            if int(page.min()) < 0:
+                raise RuntimeError("a token of this step has no page")
+            off = pos % view.page_size
+            latent_pages[page, off] = rms(x[:, q_rank:q_rank + kv_rank], kv_weight).to(latent_pages.dtype)
+            turned = self._turn(x[:, q_rank + kv_rank:q_rank + kv_rank + rot], pos, freqs)
+            rotated_pages[page, off] = turned.to(rotated_pages.dtype)
+        return c_q
+
+    def batched_linear(self, x, w, alpha=1.0, out_f32=False):
+        """`out[t, h, :] = alpha * w[h] x[t, h, :]`: x `[T, H, K]` (a view whose last axis is dense), w `[H, N, K]`."""
+        y = torch.einsum("thk,hnk->thn", x.to(w.dtype).float(), w.float()) * alpha
+        return (y if out_f32 else y.to(self.dtype)).contiguous()
+
+    def latent_attention(self, q, q_lat, num_heads, head_size, rot, kv_rank, freqs, scale, ctx, view, latent_pages,
+                         rotated_pages, window=None):
+        """For every token and head: scores q_lat . c[j] + scale * turn(q_r) . k_r[j] over the cached tokens j
+        of its request with j <= position (and position - j < window), softmax, and the weighted sum of the
+        c[j]: `[T, H, kv_rank]`. `q` `[T, H * (head_size + rot)]` holds q_r, unturned and unscaled, behind
+        each head's `head_size` elements; `q_lat` `[T, H, kv_rank]` is scaled already."""
+        t = q.shape[0]
+        ps = view.page_size
+        out = torch.empty(t, num_heads, kv_rank, dtype=torch.float32, device=q.device)
+        q_r = q.view(t, num_heads, head_size + rot)[:, :, head_size:].float()
+        q_r = self._turn(q_r, ctx.positions.long(), freqs) * scale
+        starts = ctx.run_start.tolist()
+        for r in range(ctx.num_requests):
+            s, e = starts[r], starts[r + 1]
+            if e == s:
+                continue
+            total = int(ctx.cached_lens_host[r]) + (e - s)
+            nb = -(-total // ps)
+            pages = view.block_table[r, :nb].long().clamp(min=0)
+            c = latent_pages[pages].float().reshape(nb * ps, kv_rank)[:total]
+            k_r = rotated_pages[pages].float().reshape(nb * ps, rot)[:total]
+            scores = torch.einsum("ihd,jd->hij", q_lat[s:e].float(), c) + torch.einsum("ihd,jd->hij", q_r[s:e], k_r)
+            pos = ctx.positions[s:e].long().unsqueeze(1)
+            j = torch.arange(total, device=q.device).unsqueeze(0)
+            allowed = j <= pos
+            if window is not None:
+                allowed &= pos - j < window
+            scores = scores.masked_fill(~allowed.unsqueeze(0), float("-inf"))
+            p = torch.softmax(scores, dim=-1)
+            p = torch.where(allowed.unsqueeze(0), p, torch.zeros_like(p))
+            # pages that were given back may hold anything: what the mask hides must not reach the sum
+            c = torch.where(torch.isfinite(c), c, torch.zeros_like(c))
+            out[s:e] = torch.einsum("hij,jd->ihd", p, c)
+        return out.to(self.dtype)
+
     # ---------------------------------------------------------------- output end
 
     def gather_rows(self, x, rows):

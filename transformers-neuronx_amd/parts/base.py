@@ -61,6 +61,13 @@ class Part:
         self.ops = ops
         self.dtype = dtype
 
+    def state_need(self) -> Optional["CacheNeed"]:
+        """What a part other than a mixer keeps per request between steps: a `CacheNeed` of kind "state", or
+        None. The model gives such a part a cache of its own: an embedding finds it as `ctx.input_state`, a
+        block as `ctx.call_state` (one for every call of the run order, so a layer that is named twice keeps
+        two)."""
+        return None
+
     def step_planners(self) -> Dict[str, Callable]:
         """{name: planner} of what this part's kernels want laid out with every step's integers
         (`engine.batch`): `fn(run_lens, cached, page_size) -> ({name: int32 array}, {name: host value})`."""
@@ -175,6 +182,11 @@ class Block(Part):
         self.mixer_norm = mixer_norm
         self.feed_forward_norm = feed_forward_norm
 
+    def param_decls(self, prefix: str) -> List[ParamDecl]:
+        """Tensors of the arrangement itself (norms after a part, a convolution before it, ...), named from the
+        layer's prefix. The four parts declare their own."""
+        return []
+
     def after_load(self) -> None:
         """Called when the four parts have their tensors."""
 
@@ -185,9 +197,13 @@ class Block(Part):
 @dataclass
 class Stream:
     """The residual stream between layers: float32 `[T, hidden]`, and beside it a
-    copy in the compute dtype when the last part that wrote it made one."""
+    copy in the compute dtype when the last part that wrote it made one. `history`, for arrangements that
+    read what earlier layers left: float32 `[slots, T, hidden]` with `filled` slots written (slot 0 the
+    embedded tokens, slot i + 1 the result of the i-th call), or None."""
     x: "object"
     compute: Optional["object"] = None
+    history: Optional["object"] = None
+    filled: int = 0
 
 
 class _Registry:

@@ -49,3 +49,130 @@ class PostNormBlock(Block):
         t = self.feed_forward.forward(h, ctx, x)
         x, h = self.feed_forward_norm.forward(t, True, True)
         return Stream(x, h)
+
+
+@register_block("sandwich")
+class SandwichBlock(Block):
+    """A norm before and after each part, the part's normed result scaled before it joins the stream:
+
+        x = x + mult * post_norm(mixer(conv(norm(x))))        and the same for the feed-forward,
+
+    with, each optional:
+    `taps`: what a part reads, h = norm(x), is first replaced by h + conv(h), a causal convolution over the
+        request's tokens on every channel, conv(h)_t = sum_j w[:, j] h_(t - taps + 1 + j) (zeros before the
+        request's start; weights `[width, taps]`). The last taps - 1 inputs of each part are per-request state.
+    `side`: a token-keyed input after the feed-forward. With e the `dim` elements from column `offset` on of
+        the token's row of a table, g = gelu_tanh(W_gate x) * e, y = W_proj g:
+        x = x + mult * y / sqrt(mean(y^2) + eps) * weight.
+    `depth_average`: the stream that goes on is a weighted sum of what every call so far has left and of
+        the embedded tokens, sum_j w[j] X_j (j = 0 the embedded tokens, j = i + 1 this call's result, the i-th
+        of the run order), w a tensor of `depth_average` numbers. `depth_slots` is how many X the model has.
+    The sums, the norms and the state are float32.
+    """
+
+    recordable = True
+
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm, *, mixer_post_norm, feed_forward_post_norm,
+                 names, mult: float = 1.0, taps: int = 0, conv_names=None, side=None, depth_average: int = 0,
+                 depth_name=None, depth_slots: int = 0):
+        """`names`: the checkpoint's names of the two post norms, relative to the layer's prefix; `conv_names`
+        those of the two convolutions; `side`: dict(table, dim, offset, gate, proj, norm, eps, columns), `table`
+        a full tensor name (layers share it), `columns` its width, the others relative names."""
+        super().__init__(mixer, feed_forward, mixer_norm, feed_forward_norm)
+        from .base import NORMS
+        self.has_ff = not getattr(feed_forward, "absent", False)
+        self.mixer_post = NORMS.build(mixer_post_norm)
+        self.ff_post = NORMS.build(feed_forward_post_norm) if self.has_ff else None
+        self.names, self.conv_names = tuple(names), tuple(conv_names or ())
+        self.mult, self.taps = float(mult), int(taps)
+        self.side = dict(side) if side else None
+        self.depth_average, self.depth_name, self.depth_slots = int(depth_average), depth_name, int(depth_slots)
+        self.width = mixer_norm.width
+
+    def _convs(self):
+        return (1 if self.taps > 0 else 0) * (2 if self.has_ff else 1)
+
+    def state_need(self):
+        if self.taps > 1:
+            from .base import CacheNeed
+            return CacheNeed("state", state_shapes=(("inputs", (self._convs(), self.taps - 1, self.width)),))
+        return None
+
+    def param_decls(self, prefix: str):
+        from .spec import ParamDecl
+        d = self.mixer_post.param_decls(prefix + self.names[0])
+        if self.has_ff:
+            d += self.ff_post.param_decls(prefix + self.names[1])
+        for name in self.conv_names[:self._convs()]:
+            d.append(ParamDecl(prefix + name, (self.width, self.taps), "vector"))
+        if self.side:
+            s = self.side
+            d += [ParamDecl(s["table"], (s["rows"], s["columns"]), "table"),
+                  ParamDecl(prefix + s["gate"], (s["dim"], self.width)),
+                  ParamDecl(prefix + s["proj"], (self.width, s["dim"])),
+                  ParamDecl(prefix + s["norm"], (self.width,), "vector", "around_one")]
+        if self.depth_average:
+            d.append(ParamDecl(prefix + self.depth_name, (self.depth_average,), "vector", "around_one"))
+        return d
+
+    def load(self, tensors, prefix, ops, dtype) -> None:
+        super().load(tensors, prefix, ops, dtype)
+        self.mixer_post.load(tensors, prefix + self.names[0], ops, dtype)
+        if self.has_ff:
+            self.ff_post.load(tensors, prefix + self.names[1], ops, dtype)
+        self.conv_w = [tensors[prefix + name] for name in self.conv_names[:self._convs()]]
+        if self.side:
+            s = self.side
+            self.side_table = tensors[s["table"]]
+            self.side_gate = ops.prepare_weight(tensors[prefix + s["gate"]])
+            self.side_proj = ops.prepare_weight(tensors[prefix + s["proj"]])
+            self.side_norm = tensors[prefix + s["norm"]]
+        self.depth_w = tensors[prefix + self.depth_name] if self.depth_average else None
+
+    def flops_per_token(self, keys: float = 0.0) -> float:
+        return 4.0 * self.side["dim"] * self.width if self.side else 0.0
+
+    def _input(self, norm, x, which, ctx):
+        """What a part reads: the norm of the stream, with the convolution over the request's tokens."""
+        if self.taps <= 0:
+            return norm.forward(x, False, True)[1]
+        h = norm.forward(x, True, False)[0]
+        state = ctx.call_state.state["inputs"] if self.taps > 1 else None
+        return self.ops.input_conv(h, self.conv_w[which], state, which, ctx, self.dtype)
+
+    def forward(self, stream: Stream, ctx, cache) -> Stream:
+        ops = self.ops
+        x = stream.x
+        history, filled = stream.history, stream.filled
+        if self.depth_average and history is None:
+            history = x.new_empty((self.depth_slots,) + tuple(x.shape))
+            history[0].copy_(x)
+            filled = 1
+        if self.depth_average and not filled < self.depth_slots:
+            raise ValueError(f"the average over depth has {self.depth_slots} places and the run order more calls")
+        place = history[filled] if self.depth_average else None       # where this call's own result goes
+
+        h = self._input(self.mixer_norm, x, 0, ctx)
+        y = self.mixer.forward(h, ctx, cache, None)
+        last = not self.has_ff and not self.side
+        x = debug.tap("after_mixer", self.mixer_post.add_to(y, x, self.mult, place if last else None))
+        if self.has_ff:
+            h = self._input(self.feed_forward_norm, x, 1, ctx)
+            y = self.feed_forward.forward(h, ctx, None)
+            x = self.ff_post.add_to(y, x, self.mult, place if not self.side else None)
+        if self.side:
+            s = self.side
+            rows = ctx.memo.get(("table rows", s["table"]))
+            if rows is None:        # the tokens' rows, looked up once a step for all layers
+                rows = ctx.memo[("table rows", s["table"])] = ops.embed(ctx.token_ids, self.side_table, self.dtype,
+                                                                       ctx.kept_tokens)
+            g = ops.linear(ops.cast(x, self.dtype), self.side_gate, None, act="gelu_new")
+            g = ops.mul_columns(g, rows, s["offset"])
+            y = ops.linear(g, self.side_proj, None, out_f32=True)
+            x = ops.norm_add(y, self.side_norm, None, s["eps"], False, x, self.mult, place)
+        if not self.depth_average:
+            return Stream(x, None)
+        if self.depth_average != filled + 1:
+            raise ValueError(f"this call averages {self.depth_average} results and {filled + 1} are there")
+        debug.tap("own_result", x)
+        return Stream(ops.weighted_sum(history, self.depth_w, filled + 1), None, history, filled + 1)

@@ -43,6 +43,43 @@ class TokenEmbedding(Part):
         return Stream(xf, xc)
 
 
+@register_embedding("token_pair_table")
+class TokenPairEmbedding(Part):
+    """Token rows plus a row that depends on the token and the one before it in its request:
+    `x = table[token] + pairs[(previous * mul_prev + token * mul_cur) mod buckets]`, and for the first token of
+    a request the row after the buckets (the table has buckets + 1 rows). The sum is float32. A request's last
+    token is per-request state: a step's first token of a request pairs with it."""
+
+    recordable = True
+
+    def __init__(self, vocab: int, width: int, buckets: int, mul_prev: int, mul_cur: int, table_name: str,
+                 pairs_name: str):
+        self.vocab, self.width, self.buckets = vocab, width, buckets
+        self.mul_prev, self.mul_cur = mul_prev, mul_cur
+        self.table_name, self.pairs_name = table_name, pairs_name
+        self.position = POSITIONS.build(PartSpec("none", {}))
+        if buckets <= 0:
+            raise ValueError(f"a pair table needs buckets, got {buckets}")
+
+    def state_need(self):
+        from .base import CacheNeed
+        return CacheNeed("state", state_shapes=(("last_token", (1,)),), state_dtype="int32")
+
+    def param_decls(self, prefix: str = "") -> List[ParamDecl]:
+        return [ParamDecl(self.table_name, (self.vocab, self.width), "table"),
+                ParamDecl(self.pairs_name, (self.buckets + 1, self.width), "table")]
+
+    def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
+        super().load(tensors, prefix, ops, dtype)
+        self.table, self.pairs = tensors[self.table_name], tensors[self.pairs_name]
+        self.position.load(tensors, "", ops, dtype)
+
+    def forward(self, ctx, want_compute: bool) -> Stream:
+        x = self.ops.embed_pairs(ctx.token_ids, self.table, self.pairs, self.buckets, self.mul_prev, self.mul_cur,
+                                 ctx, ctx.input_state.state["last_token"], ctx.kept_tokens)
+        return Stream(x, self.ops.cast(x, self.dtype) if want_compute else None)
+
+
 @register_head("vocab_projection")
 class VocabHead(Part):
     """Rows that need logits are picked first, then an optional norm, an optional
@@ -54,7 +91,11 @@ class VocabHead(Part):
     recordable = True
 
     def __init__(self, vocab: int, embed_width: int, width: int, norm: Optional[PartSpec],
-                 weight_name: str, tied_to: Optional[str], projection_name: Optional[str], norm_name: str):
+                 weight_name: str, tied_to: Optional[str], projection_name: Optional[str], norm_name: str,
+                 logit_scale: float = 1.0):
+        """`logit_scale`: the logits are the product times this number (folded into the matrix's float32
+        result, not into the matrix)."""
+        self.logit_scale = float(logit_scale)
         self.vocab, self.embed_width, self.width = vocab, embed_width, width
         self.norm = NORMS.build(norm) if norm is not None else None
         self.weight_name, self.tied_to = weight_name, tied_to
@@ -86,4 +127,5 @@ class VocabHead(Part):
             h = self.ops.cast(rows, self.dtype)
         if self.projects:
             h = self.ops.linear(h, self.projection, None)
-        return self.ops.linear(h, self.weight, None, out_f32=True)
+        logits = self.ops.linear(h, self.weight, None, out_f32=True)
+        return logits if self.logit_scale == 1.0 else logits.mul_(self.logit_scale)

@@ -121,3 +121,111 @@ class Attention(Mixer):
         c = self.ops.attention(q, self.num_heads, self.num_kv_heads, self.head_size, ctx, view,
                                cache.k_pages, cache.v_pages, self.window)
         return self.ops.linear(c, self.w_out, self.b_out, residual=residual, out_f32=True)
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Mixer):
+    """Softmax attention whose keys and values are made from one small vector a token, and only that vector
+    is cached.
+
+    With H heads, per head n unrotated and r rotated query/key elements and v value elements, a key/value
+    latent of R and a query latent of Q elements:
+        c_q = rms_norm(W_dq h),  q = W_uq c_q  laid out head by head as [n | r]
+        [c' | k_r'] = W_dkv h,   c = rms_norm(c'),  k_r = turn(k_r')      (R and r elements; k_r is shared by the heads)
+        score(i, j, head) = scale * (q_n[i] . (W_uk c[j]) + turn(q_r[i]) . k_r[j]),   value = W_uv c[j]
+    over the keys of the query's own request at positions j <= i (and i - j < window with a window), softmax
+    in float32, then W_o on the heads side by side. `turn` is the `rotation` (a `rotary` position part).
+
+    The cache holds c and k_r, in pages of their own shapes. The products with W_uk and W_uv are moved to the
+    query's side, so that a cached token is read as it lies: q_lat = scale * W_uk^T q_n (R elements a head),
+    score = q_lat . c + scale * q_r . k_r, and the weighted sum of the c[j] goes through W_uv afterwards.
+
+    `own_kv=False`: no W_dkv; the mixer reads the cache of another call of the run order, whose R, r and
+    rotation are its own. `keep`: the tokens the cache keeps (None: all); a cache that is read by mixers of
+    different windows keeps the most any of them sees.
+    """
+
+    recordable = True
+
+    def __init__(self, width: int, num_heads: int, head_size: int, rot_size: int, value_size: int, kv_rank: int,
+                 q_rank: int, scale: float, eps: float, rotation, names, window: Optional[int] = None,
+                 keep: Optional[int] = None, own_kv: bool = True, norm_suffix: str = ".norm", weight_suffix: str = ""):
+        """`names`: the checkpoint's names, relative to the mixer's prefix, of W_dq, W_uq, W_dkv, W_uk, W_uv and
+        W_o; a latent's norm weight is its down-projection's name with `norm_suffix`."""
+        self.width, self.num_heads, self.head_size, self.rot_size = width, num_heads, head_size, rot_size
+        self.value_size, self.kv_rank, self.q_rank = value_size, kv_rank, q_rank
+        self.scale, self.eps, self.window, self.own_kv = float(scale), float(eps), window, own_kv
+        self.keep = keep if own_kv else None
+        if own_kv and window is not None and keep is not None and keep < window:
+            raise ValueError(f"a cache that keeps {keep} tokens cannot serve a window of {window}")
+        self.names = tuple(names)
+        if len(self.names) != 6:
+            raise ValueError("names: W_dq, W_uq, W_dkv, W_uk, W_uv, W_o, six names")
+        self.norm_suffix, self.weight_suffix = norm_suffix, weight_suffix
+        self.rotation = POSITIONS.build(rotation)
+        if rot_size % 2 or self.rotation.dims > rot_size:
+            raise ValueError(f"the rotated part has {rot_size} elements; the rotation turns {self.rotation.dims}")
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        keep = self.keep if self.keep is not None else self.window
+        return CacheNeed("paged", window=keep,
+                         page_tensors=(("latent", ("page", self.kv_rank)), ("rotated", ("page", self.rot_size))))
+
+    def param_decls(self, prefix: str) -> List[ParamDecl]:
+        dq, uq, dkv, uk, uv, o = (prefix + n for n in self.names)
+        s, h = self.weight_suffix, self.num_heads
+        d = [ParamDecl(dq + s, (self.q_rank, self.width)),
+             ParamDecl(dq + self.norm_suffix, (self.q_rank,), "vector", "around_one"),
+             ParamDecl(uq + s, (h * (self.head_size + self.rot_size), self.q_rank))]
+        if self.own_kv:
+            d += [ParamDecl(dkv + s, (self.kv_rank + self.rot_size, self.width)),
+                  ParamDecl(dkv + self.norm_suffix, (self.kv_rank,), "vector", "around_one")]
+        d += [ParamDecl(uk + s, (h * self.head_size, self.kv_rank)),
+              ParamDecl(uv + s, (h * self.value_size, self.kv_rank)),
+              ParamDecl(o + s, (self.width, h * self.value_size))]
+        return d
+
+    def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
+        super().load(tensors, prefix, ops, dtype)
+        dq, uq, dkv, uk, uv, o = (prefix + n for n in self.names)
+        s, h = self.weight_suffix, self.num_heads
+        # one product for both latents: the rows of W_dq, then those of W_dkv
+        down = [tensors[dq + s]] + ([tensors[dkv + s]] if self.own_kv else [])
+        self.w_down = ops.prepare_weight(torch.cat(down, dim=0).contiguous())
+        self.q_norm = tensors[dq + self.norm_suffix]
+        self.kv_norm = tensors[dkv + self.norm_suffix] if self.own_kv else None
+        self.w_uq = ops.prepare_weight(tensors[uq + s])
+        # W_uk a head, transposed: [H, R, n], the matrix that takes a head's q_n to its q_lat
+        self.w_uk_t = tensors[uk + s].view(h, self.head_size, self.kv_rank).transpose(1, 2).contiguous()
+        self.w_uv = tensors[uv + s].view(h, self.value_size, self.kv_rank).contiguous()
+        self.w_o = ops.prepare_weight(tensors[o + s])
+        self.rotation.load(tensors, prefix + "rotation", ops, dtype)
+        self.freqs = self.rotation.frequencies()
+        if not self.rotation.interleaved:
+            raise ValueError("latent attention turns neighbouring pairs (the interleaved layout)")
+
+    def first_weight(self):
+        return None          # the product's float32 result goes to two norms: the norm before it stays a kernel
+
+    def flops_per_token(self, keys: float = 0.0) -> float:
+        seen = min(keys, self.window) if self.window else keys
+        return super().flops_per_token(keys) + 2.0 * self.num_heads * (2 * self.kv_rank + self.rot_size) * seen
+
+    def forward(self, h, ctx, cache, residual):
+        if cache.writes != self.own_kv:
+            raise ValueError("a latent-attention mixer with own_kv writes its cache; one without reads another's")
+        ops, view = self.ops, ctx.groups[cache.group]
+        heads, n, r = self.num_heads, self.head_size, self.rot_size
+        latent, rotated = cache.pages["latent"], cache.pages["rotated"]
+        if latent.shape[-1] != self.kv_rank or rotated.shape[-1] != r:
+            raise ValueError(f"the cache holds latents of {latent.shape[-1]} + {rotated.shape[-1]} elements, "
+                             f"this mixer reads {self.kv_rank} + {r}")
+        down = ops.linear(h, self.w_down, None, out_f32=True)
+        c_q = ops.latent_norms(down, self.q_rank, self.kv_rank if self.own_kv else 0, r if self.own_kv else 0,
+                               self.q_norm, self.kv_norm, self.eps, self.freqs, ctx, view, latent, rotated)
+        q = ops.linear(c_q, self.w_uq, None)
+        q_lat = ops.batched_linear(q.view(-1, heads, n + r)[:, :, :n], self.w_uk_t, alpha=self.scale)
+        o_lat = ops.latent_attention(q, q_lat, heads, n, r, self.kv_rank, self.freqs, self.scale, ctx, view,
+                                     latent, rotated, self.window)
+        values = ops.batched_linear(o_lat, self.w_uv)
+        return ops.linear(values.view(-1, heads * self.value_size), self.w_o, None, residual=residual, out_f32=True)

@@ -13,27 +13,64 @@ class LayerNorm(Norm):
 
     recordable = True
 
-    def __init__(self, width: int, eps: float, affine: bool = True):
+    def __init__(self, width: int, eps: float, affine: bool = True, weight_suffix: str = ".weight",
+                 bias_suffix: str = ".bias"):
+        """`weight_suffix`, `bias_suffix`: what the checkpoint's names of the two vectors add to the norm's."""
         self.width, self.eps, self.affine = width, float(eps), affine
+        self.weight_suffix, self.bias_suffix = weight_suffix, bias_suffix
         self.weight = self.bias = None
 
     def param_decls(self, prefix: str) -> List[ParamDecl]:
         if not self.affine:
             return []
-        return [ParamDecl(prefix + ".weight", (self.width,), "vector", "around_one"),
-                ParamDecl(prefix + ".bias", (self.width,), "vector", "normal")]
+        return [ParamDecl(prefix + self.weight_suffix, (self.width,), "vector", "around_one"),
+                ParamDecl(prefix + self.bias_suffix, (self.width,), "vector", "normal")]
 
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
         super().load(tensors, prefix, ops, dtype)
         if self.affine:
-            self.weight = tensors[prefix + ".weight"]
-            self.bias = tensors[prefix + ".bias"]
+            self.weight = tensors[prefix + self.weight_suffix]
+            self.bias = tensors[prefix + self.bias_suffix]
 
     def forward(self, x, want_f32: bool, want_compute: bool):
         return self.ops.layernorm(x, self.weight, self.bias, self.eps, self.dtype, want_f32, want_compute)
+
+    def add_to(self, y, residual, mult: float = 1.0, out=None):
+        """`residual + mult * norm(y)` in float32 (into `out`, if given): the norm that follows a part."""
+        return self.ops.norm_add(y, self.weight, self.bias, self.eps, True, residual, mult, out)
 
     def fold_into(self, w) -> bool:
         return self.ops.fold_norm(w, self.weight, self.bias)
 
     def deferred(self, x):
         return self.ops.layernorm_deferred(x, self.weight, self.bias, self.eps, self.dtype)
+
+
+@register_norm("rms_norm")
+class RMSNorm(Norm):
+    """`x / sqrt(mean(x^2) + eps) * weight`, statistics in float32: the norm that only scales."""
+
+    recordable = True
+
+    def __init__(self, width: int, eps: float, weight_suffix: str = ".weight"):
+        self.width, self.eps, self.weight_suffix = width, float(eps), weight_suffix
+        self.weight = None
+
+    def param_decls(self, prefix: str) -> List[ParamDecl]:
+        return [ParamDecl(prefix + self.weight_suffix, (self.width,), "vector", "around_one")]
+
+    def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
+        super().load(tensors, prefix, ops, dtype)
+        self.weight = tensors[prefix + self.weight_suffix]
+
+    def forward(self, x, want_f32: bool, want_compute: bool):
+        return self.ops.layernorm(x, self.weight, None, self.eps, self.dtype, want_f32, want_compute, center=False)
+
+    def add_to(self, y, residual, mult: float = 1.0, out=None):
+        return self.ops.norm_add(y, self.weight, None, self.eps, False, residual, mult, out)
+
+    def fold_into(self, w) -> bool:
+        return self.ops.fold_norm(w, self.weight, None, center=False)
+
+    def deferred(self, x):
+        return self.ops.layernorm_deferred(x, self.weight, None, self.eps, self.dtype, center=False)

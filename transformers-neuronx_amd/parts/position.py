@@ -40,3 +40,47 @@ class NoPositions(PositionEncoding):
 
     def at_input(self, x, positions, want_compute: bool):
         return self.ops.to_stream(x, self.dtype, want_compute)
+
+
+@register_position("rotary")
+class RotaryPositions(PositionEncoding):
+    """Turns pairs of query and key elements by an angle that grows with the position: of the first `dims`
+    elements of a head, element 2i is paired with 2i + 1 (`interleaved`) or element i with i + dims / 2, and the
+    pair (u, v) at position p becomes (u cos a - v sin a, v cos a + u sin a), a = p * base^(-2i / dims). The
+    elements beyond `dims` pass. Positions, frequencies and angles are float32.
+
+    Two ways to use it: `pair_tables` (the attention mixer's pairwise form, for `max_positions` positions,
+    interleaved pairs only), or `frequencies()`, for a mixer whose kernels make the angles themselves."""
+
+    recordable = True
+
+    def __init__(self, base: float, dims: int, max_positions: int = 0, interleaved: bool = True):
+        if dims % 2 or dims < 0:
+            raise ValueError(f"rotary positions turn pairs: dims must be even, got {dims}")
+        self.base, self.dims, self.max_positions, self.interleaved = float(base), dims, max_positions, interleaved
+        self.device = "cpu"
+
+    def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
+        super().load(tensors, prefix, ops, dtype)
+        self.device = getattr(ops, "device", "cpu")
+        self._freqs = None
+
+    def frequencies(self):
+        """float32 `[dims / 2]` on the device: base^(-2i / dims), made in float64 and rounded once."""
+        if getattr(self, "_freqs", None) is None:
+            import torch
+            i = torch.arange(self.dims // 2, dtype=torch.float64)
+            self._freqs = (self.base ** (-2.0 * i / max(self.dims, 1))).to(torch.float32).to(self.device)
+        return self._freqs
+
+    def pair_tables(self, head_size: int):
+        import torch
+        if not self.interleaved or self.max_positions <= 0 or self.dims > head_size:
+            return None
+        angle = torch.arange(self.max_positions, dtype=torch.float32)[:, None] * self.frequencies().cpu()[None, :]
+        cos, sin = torch.cos(angle), torch.sin(angle)
+        a = torch.ones(self.max_positions, head_size, dtype=torch.float32)
+        b = torch.zeros(self.max_positions, head_size, dtype=torch.float32)
+        a[:, :self.dims] = torch.stack([cos, cos], dim=-1).reshape(self.max_positions, self.dims)
+        b[:, :self.dims] = torch.stack([-sin, sin], dim=-1).reshape(self.max_positions, self.dims)
+        return a.contiguous().to(self.device), b.contiguous().to(self.device)

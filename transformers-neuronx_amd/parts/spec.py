@@ -85,6 +85,9 @@ class ModelSpec:
     # A checkpoint of the base model alone names its tensors without this leading piece; the loader
     # tries a declared name without it when the name itself is absent ("" : no such form).
     base_model_prefix: str = ""
+    # Tensors a checkpoint may hold that this model does not read (a layer built without one of its parts
+    # whose file still carries that part's vectors): the loader passes over them instead of refusing the file.
+    unread: Tuple[str, ...] = ()
 
     @staticmethod
     def sequential(n_layers: int) -> Tuple[LayerCall, ...]:

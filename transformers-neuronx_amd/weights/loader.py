@@ -144,12 +144,13 @@ def resolve_names(decls: Iterable[ParamDecl], source, base_prefix: str = "") -> 
     return out
 
 
-def check(decls: List[ParamDecl], source, base_prefix: str = "") -> Dict[str, Optional[str]]:
+def check(decls: List[ParamDecl], source, base_prefix: str = "", unread: Iterable[str] = ()) -> Dict[str, Optional[str]]:
     """Raise one `WeightsError` for everything that is wrong; return the name map."""
     names = resolve_names(decls, source, base_prefix)
     missing = [n for n, src in names.items() if src is None]
     used = {src for src in names.values() if src is not None}
     declared = {d.name for d in decls} | {b for d in decls if (b := _base_model_name(d.name, base_prefix))}
+    declared |= set(unread)
     unexpected = [n for n in source.names() if n not in used and n not in declared]
     wrong_shape, wrong_dtype = [], []
     for d in decls:
@@ -189,10 +190,10 @@ def target_dtype(role: str, stored: torch.dtype, compute: torch.dtype, cast_floa
 
 
 def load_tensors(decls: List[ParamDecl], source, compute: torch.dtype, device, base_prefix: str = "",
-                 cast_float32: bool = False) -> Dict[str, torch.Tensor]:
+                 cast_float32: bool = False, unread: Iterable[str] = ()) -> Dict[str, torch.Tensor]:
     """Check, then read every declared tensor to `device` in its target dtype.
     Tensors that resolve to the same source tensor share one device buffer."""
-    names = check(decls, source, base_prefix)
+    names = check(decls, source, base_prefix, unread)
     by_source: Dict[tuple, torch.Tensor] = {}
     out = {}
     kept_wide, halves = [], []
