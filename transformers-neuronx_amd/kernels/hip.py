@@ -79,6 +79,28 @@ _SIGNATURES = {
         "tnx_sample": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                        _c_int, _c_void_p],
     },
+    "stream": {
+        "tnx_embed_pairs": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_ll, _c_ll,
+                            _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                            _c_void_p],
+        "tnx_norm_add": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_float, _c_void_p, _c_int,
+                         _c_int, _c_void_p],
+        "tnx_input_conv": [_c_void_p, _c_void_p, _c_void_p, _c_ll, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                           _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_poly_norm": [_c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_mul_columns": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_void_p],
+        "tnx_weighted_sum": [_c_void_p, _c_void_p, _c_int, _c_ll, _c_void_p, _c_ll, _c_void_p],
+    },
+    "latent": {
+        "tnx_latent_norms": [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int,
+                             _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_ll, _c_ll,
+                             _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_batched_linear": [_c_void_p, _c_int, _c_ll, _c_ll, _c_void_p, _c_int, _c_void_p, _c_int, _c_float, _c_int,
+                               _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_latent_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                                     _c_int, _c_int, _c_void_p, _c_void_p, _c_ll, _c_ll, _c_void_p, _c_int, _c_float,
+                                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    },
     "probe": {
         "tnx_probe_stream_read": [_c_void_p, ctypes.c_size_t, _c_void_p, _c_int, _c_void_p],
         "tnx_probe_mfma_loop": [_c_int, _c_int, _c_void_p, _c_void_p],
@@ -970,6 +992,158 @@ class HipOps:
         blocks = self._decode_blocks(num_heads, num_kv_heads or num_heads, head_size)
         return ("decode", blocks, head_size) + self._splits_for(step.length_bound, fills, alike, n_dec * blocks,
                                                                 int(window or 0), head_size)
+
+    # ---------------------------------------------------------------- parts of other designs
+
+    def embed_pairs(self, token_ids, table, pairs, buckets, mul_prev, mul_cur, ctx, last_token, kept_tokens=None):
+        """See `ReferenceOps.embed_pairs`."""
+        t = token_ids.numel()
+        _want(token_ids, "token ids", torch.int32)
+        _want(table, "token table")
+        _want(pairs, "pair table", table.dtype, (buckets + 1, table.shape[1]))
+        _want(last_token, "last tokens", torch.int32)
+        if last_token.dim() != 2 or last_token.shape[1] != 2:
+            raise ValueError(f"last tokens are [slots, 2], got {tuple(last_token.shape)}")
+        if kept_tokens is not None:
+            _want(kept_tokens, "kept tokens", torch.int32)
+        out = torch.empty(t, table.shape[1], dtype=torch.float32, device=table.device)
+        self._call("stream", "tnx_embed_pairs", _ptr(token_ids), _ptr(kept_tokens),
+                   kept_tokens.numel() if kept_tokens is not None else 0, _ptr(table), _ptr(pairs), _code(table.dtype),
+                   table.shape[0], buckets, mul_prev, mul_cur, _ptr(ctx.positions), _ptr(ctx.token_request),
+                   _ptr(ctx.run_start), _ptr(ctx.slots), _ptr(last_token), _ptr(out), t, table.shape[1],
+                   ctx.num_requests, _stream())
+        return out
+
+    def norm_add(self, y, weight, bias, eps, center, residual, mult=1.0, out=None):
+        """float32 `residual + mult * norm(y)`; `center` as in `layernorm`."""
+        _want(y, "y", torch.float32)
+        t, width = y.shape
+        _want(residual, "residual", torch.float32, (t, width))
+        if weight is not None:
+            _want(weight, "norm weight", torch.float32, (width,))
+        if bias is not None:
+            _want(bias, "norm bias", torch.float32, (width,))
+        if out is None:
+            out = torch.empty_like(y)
+        else:
+            _want(out, "out", torch.float32, (t, width))
+        self._call("stream", "tnx_norm_add", _ptr(y), _ptr(weight), _ptr(bias), float(eps), int(bool(center)),
+                   _ptr(residual), float(mult), _ptr(out), t, width, _stream())
+        return out
+
+    def input_conv(self, h, weight, state, which, ctx, dtype):
+        """See `ReferenceOps.input_conv`."""
+        _want(h, "h", torch.float32)
+        t, width = h.shape
+        taps = weight.shape[1]
+        _want(weight, "convolution weights", torch.float32, (width, taps))
+        mine, stride = None, 0
+        if taps > 1:
+            _want(state, "convolution state", torch.float32)
+            if state.dim() != 4 or tuple(state.shape[2:]) != (taps, width) or not 0 <= which < state.shape[1]:
+                raise ValueError(f"convolution state is [slots, parts, {taps}, {width}], got {tuple(state.shape)}")
+            mine, stride = state.data_ptr() + which * taps * width * 4, state.stride(0)
+        out = torch.empty(t, width, dtype=dtype, device=h.device)
+        self._call("stream", "tnx_input_conv", _ptr(h), _ptr(weight), mine, stride, taps, _ptr(ctx.positions),
+                   _ptr(ctx.token_request), _ptr(ctx.run_start), _ptr(ctx.slots), _ptr(out), _code(dtype), t, width, ctx.num_requests, _stream())
+        return out
+
+    def poly_norm(self, z, coeffs, eps):
+        """See `ReferenceOps.poly_norm`."""
+        _want(z, "z", torch.float32)
+        _want(coeffs, "coefficients", torch.float32, (4,))
+        out = torch.empty(z.shape, dtype=self.dtype, device=z.device)
+        self._call("stream", "tnx_poly_norm", _ptr(z), _ptr(coeffs), float(eps), _ptr(out), _code(self.dtype),
+                   z.shape[0], z.shape[1], _stream())
+        return out
+
+    def mul_columns(self, g, rows, offset):
+        _want(g, "g", self.dtype)
+        _want(rows, "rows", self.dtype)
+        if rows.shape[0] != g.shape[0]:
+            raise ValueError(f"{g.shape[0]} rows of g, {rows.shape[0]} rows of the table")
+        out = torch.empty_like(g)
+        self._call("stream", "tnx_mul_columns", _ptr(g), _ptr(rows), _code(self.dtype), int(offset), g.shape[1],
+                   rows.shape[1], _ptr(out), g.shape[0], _stream())
+        return out
+
+    def weighted_sum(self, history, weights, count):
+        _want(history, "history", torch.float32)
+        _want(weights, "weights", torch.float32)
+        if not 1 <= count <= history.shape[0] or weights.numel() < count:
+            raise ValueError(f"weighted_sum of {count} slots: {history.shape[0]} are there, {weights.numel()} weights")
+        out = torch.empty_like(history[0])
+        self._call("stream", "tnx_weighted_sum", _ptr(history), _ptr(weights), count, history.stride(0), _ptr(out),
+                   out.numel(), _stream())
+        return out
+
+    def _latent_pages(self, latent_pages, rotated_pages, kv_rank, rot, page_size):
+        for pages, name, last in ((latent_pages, "latent pages", kv_rank), (rotated_pages, "rotated pages", rot)):
+            if not pages.is_cuda or pages.dtype != self.dtype:
+                raise TypeError(f"{name} must be {self.dtype} on the GPU, got {pages.dtype} on {pages.device}")
+            if pages.dim() != 3 or tuple(pages.shape[1:]) != (page_size, last) or tuple(pages.stride()[1:]) != (last, 1) \
+                    or pages.stride(0) < page_size * last:
+                raise ValueError(f"{name} are [pages, {page_size}, {last}] with a page's elements together, got "
+                                 f"{tuple(pages.shape)} with strides {tuple(pages.stride())}")
+        if latent_pages.shape[0] != rotated_pages.shape[0]:
+            raise ValueError("latent and rotated pages differ in number")
+        return latent_pages.shape[0]
+
+    def latent_norms(self, down, q_rank, kv_rank, rot, q_weight, kv_weight, eps, freqs, ctx, view, latent_pages,
+                     rotated_pages):
+        """See `ReferenceOps.latent_norms`."""
+        t = ctx.num_tokens
+        _want(down, "down", torch.float32, (t, q_rank + kv_rank + rot))
+        _want(q_weight, "query latent norm", torch.float32, (q_rank,))
+        _want(freqs, "frequencies", torch.float32)
+        num_pages = 0
+        if kv_rank:
+            _want(kv_weight, "key/value latent norm", torch.float32, (kv_rank,))
+            num_pages = self._latent_pages(latent_pages, rotated_pages, kv_rank, rot, view.page_size)
+            _want(view.token_page, "token pages", torch.int32, (t,))
+            _want(view.token_offset, "token offsets", torch.int32, (t,))
+        c_q = torch.empty(t, q_rank, dtype=self.dtype, device=down.device)
+        self._call("latent", "tnx_latent_norms", _ptr(down), q_rank, kv_rank, rot, _ptr(q_weight), _ptr(kv_weight),
+                   float(eps), _ptr(freqs), freqs.numel(), _ptr(ctx.positions), _ptr(view.token_page),
+                   _ptr(view.token_offset), _ptr(c_q), _code(self.dtype), _ptr(latent_pages) if kv_rank else None,
+                   _ptr(rotated_pages) if kv_rank else None, latent_pages.stride(0) if kv_rank else 0,
+                   rotated_pages.stride(0) if kv_rank else 0, num_pages, view.page_size, t, _stream())
+        return c_q
+
+    def batched_linear(self, x, w, alpha=1.0, out_f32=False):
+        """`out[t, h, :] = alpha * w[h] x[t, h, :]`: x `[T, H, K]` (a view whose last axis is dense), w `[H, N, K]`."""
+        if x.dim() != 3 or w.dim() != 3 or x.shape[1] != w.shape[0] or x.shape[2] != w.shape[2]:
+            raise ValueError(f"batched_linear: x {tuple(x.shape)} does not fit w {tuple(w.shape)}")
+        if not x.is_cuda or x.stride(2) != 1:
+            raise ValueError("batched_linear: x must be on the GPU with a dense last axis")
+        _want(w, "w")
+        t, heads, k = x.shape
+        n = w.shape[1]
+        out = torch.empty(t, heads, n, dtype=torch.float32 if out_f32 else self.dtype, device=x.device)
+        self._call("latent", "tnx_batched_linear", _ptr(x), _code(x.dtype), x.stride(0), x.stride(1), _ptr(w),
+                   _code(w.dtype), _ptr(out), _code(out.dtype), float(alpha), t, heads, n, k, _stream(),
+                   work=(f"{t}x{heads}x{n}x{k}", heads * n * k * w.element_size() + t * heads * (k + n) * 2,
+                         2.0 * t * heads * n * k))
+        return out
+
+    def latent_attention(self, q, q_lat, num_heads, head_size, rot, kv_rank, freqs, scale, ctx, view, latent_pages,
+                         rotated_pages, window=None):
+        """See `ReferenceOps.latent_attention`."""
+        t = ctx.num_tokens
+        _want(q, "q", self.dtype, (t, num_heads * (head_size + rot)))
+        _want(q_lat, "q_lat", self.dtype, (t, num_heads, kv_rank))
+        _want(freqs, "frequencies", torch.float32)
+        num_pages = self._latent_pages(latent_pages, rotated_pages, kv_rank, rot, view.page_size)
+        _want(view.block_table, "block table", torch.int32, (ctx.num_requests, view.width))
+        if ctx.max_total > view.width * view.page_size:
+            raise ValueError("a request is longer than its block table")
+        out = torch.empty(t, num_heads, kv_rank, dtype=self.dtype, device=q.device)
+        self._call("latent", "tnx_latent_attention_any", _ptr(q), _code(self.dtype), _ptr(q_lat), _ptr(out),
+                   _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
+                   num_pages, _ptr(latent_pages), _ptr(rotated_pages), latent_pages.stride(0), rotated_pages.stride(0),
+                   _ptr(freqs), freqs.numel(), float(scale), num_heads, head_size, rot, kv_rank, int(window or 0), t,
+                   _stream())
+        return out
 
     # ---------------------------------------------------------------- output end
 

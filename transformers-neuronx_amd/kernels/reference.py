@@ -196,18 +196,19 @@ class ReferenceOps:
 
     def embed_pairs(self, token_ids, table, pairs, buckets, mul_prev, mul_cur, ctx, last_token, kept_tokens=None):
         """float32 `table[token] + pairs[row]`, row = (previous * mul_prev + token * mul_cur) mod buckets, and
-        `buckets` at position 0; the token before a step's first of a request is `last_token[slot, 0]`, which
-        then takes the request's last token of this step."""
+        `buckets` at position 0. `last_token` `[slots, 2]` keeps a request's last token at place (its position) & 1:
+        the token before a step's first of a request is read there, and the step's last is written."""
         ids = self._resolved(token_ids, kept_tokens)
         starts = ctx.run_start.long()
         first = torch.zeros_like(ids, dtype=torch.bool)
         first[starts[:-1]] = True
         slots = ctx.slots.long()
         before = torch.roll(ids, 1)
-        before[starts[:-1]] = last_token[slots, 0].long()
+        pos = ctx.positions.long()
+        before[starts[:-1]] = last_token[slots, (pos[starts[:-1]] - 1) & 1].long()
         rows = (before * mul_prev + ids * mul_cur) % buckets
         rows = torch.where(ctx.positions.long() == 0, torch.full_like(rows, buckets), rows)
-        last_token[slots, 0] = ids[starts[1:] - 1].to(last_token.dtype)
+        last_token[slots, pos[starts[1:] - 1] & 1] = ids[starts[1:] - 1].to(last_token.dtype)
         return table[ids].float() + pairs[rows].float()
 
     def norm_add(self, y, weight, bias, eps, center, residual, mult=1.0, out=None):
@@ -222,16 +223,20 @@ class ReferenceOps:
     def input_conv(self, h, weight, state, which, ctx, dtype):
         """`h + conv(h)`: conv(h)_t = sum_j weight[:, j] h_(t - taps + 1 + j) over the tokens of t's own request;
         the taps - 1 inputs before a step's first token of a request come from `state[slot, which]`
-        (`[taps - 1, width]`, oldest first, zeros at a request's start), which then takes the last ones."""
+        (`[taps, width]`: the input at position p at place p mod taps; zeros before a request's start), which
+        then takes the run's last ones."""
         taps = weight.shape[1]
         out = torch.empty_like(h)
         start = 0
         for r in range(ctx.num_requests):
-            n, slot = int(ctx.run_lens_host[r]), int(ctx.slots_host[r])
+            n, slot, have = int(ctx.run_lens_host[r]), int(ctx.slots_host[r]), int(ctx.cached_lens_host[r])
             run = h[start:start + n].float()
             if taps > 1:
-                seq = torch.cat([state[slot, which].float(), run], dim=0)
-                state[slot, which] = seq[-(taps - 1):]
+                before = [state[slot, which, p % taps].float() if p >= 0 else torch.zeros_like(run[0])
+                          for p in range(have - (taps - 1), have)]
+                seq = torch.cat([torch.stack(before), run], dim=0)
+                for i in range(max(0, n - (taps - 1)), n):
+                    state[slot, which, (have + i) % taps] = run[i]
             else:
                 seq = run
             acc = run.clone()

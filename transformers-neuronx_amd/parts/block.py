@@ -60,7 +60,8 @@ class SandwichBlock(Block):
     with, each optional:
     `taps`: what a part reads, h = norm(x), is first replaced by h + conv(h), a causal convolution over the
         request's tokens on every channel, conv(h)_t = sum_j w[:, j] h_(t - taps + 1 + j) (zeros before the
-        request's start; weights `[width, taps]`). The last taps - 1 inputs of each part are per-request state.
+        request's start; weights `[width, taps]`). The last taps - 1 inputs of each part are per-request state
+        (kept in `taps` places, by position, so that a step of single tokens can be run again and read the same).
     `side`: a token-keyed input after the feed-forward. With e the `dim` elements from column `offset` on of
         the token's row of a table, g = gelu_tanh(W_gate x) * e, y = W_proj g:
         x = x + mult * y / sqrt(mean(y^2) + eps) * weight.
@@ -95,7 +96,7 @@ class SandwichBlock(Block):
     def state_need(self):
         if self.taps > 1:
             from .base import CacheNeed
-            return CacheNeed("state", state_shapes=(("inputs", (self._convs(), self.taps - 1, self.width)),))
+            return CacheNeed("state", state_shapes=(("inputs", (self._convs(), self.taps, self.width)),))
         return None
 
     def param_decls(self, prefix: str):

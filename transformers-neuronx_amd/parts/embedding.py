@@ -48,7 +48,8 @@ class TokenPairEmbedding(Part):
     """Token rows plus a row that depends on the token and the one before it in its request:
     `x = table[token] + pairs[(previous * mul_prev + token * mul_cur) mod buckets]`, and for the first token of
     a request the row after the buckets (the table has buckets + 1 rows). The sum is float32. A request's last
-    token is per-request state: a step's first token of a request pairs with it."""
+    token is per-request state (two places, by the parity of its position): a step's first token of a request
+    pairs with it."""
 
     recordable = True
 
@@ -63,7 +64,7 @@ class TokenPairEmbedding(Part):
 
     def state_need(self):
         from .base import CacheNeed
-        return CacheNeed("state", state_shapes=(("last_token", (1,)),), state_dtype="int32")
+        return CacheNeed("state", state_shapes=(("last_token", (2,)),), state_dtype="int32")
 
     def param_decls(self, prefix: str = "") -> List[ParamDecl]:
         return [ParamDecl(self.table_name, (self.vocab, self.width), "table"),
