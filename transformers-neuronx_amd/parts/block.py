@@ -113,7 +113,7 @@ class SandwichBlock(Block):
                   ParamDecl(prefix + s["proj"], (self.width, s["dim"])),
                   ParamDecl(prefix + s["norm"], (self.width,), "vector", "around_one")]
         if self.depth_average:
-            d.append(ParamDecl(prefix + self.depth_name, (self.depth_average,), "vector", "around_one"))
+            d.append(ParamDecl(prefix + self.depth_name, (self.depth_average,), "vector", "around_mean"))
         return d
 
     def load(self, tensors, prefix, ops, dtype) -> None:
