@@ -161,15 +161,17 @@ def test_latent_norms_and_their_pages(name, dtype, tol):
     freqs = (50.0 ** (-2.0 * torch.arange(pairs, dtype=torch.float64) / (2 * pairs))).float()
     lat = torch.zeros(5, ps, R, dtype=dtype, device=DEV)
     rot = torch.zeros(5, ps, r, dtype=dtype, device=DEV)
+    across = torch.zeros(5, R, ps, dtype=dtype, device=DEV)
     # one request of 9 tokens from position 12 on: crosses from page 3 into page 1
     ctx = _ctx([9], [12], [0], {"g": [[3, 1, 4]]}, ps)
-    c_q = ops.latent_norms(down.to(DEV), Q, R, r, qw.to(DEV), kw.to(DEV), 1e-5, freqs.to(DEV), ctx, ctx.groups["g"], lat, rot)
+    c_q = ops.latent_norms(down.to(DEV), Q, R, r, qw.to(DEV), kw.to(DEV), 1e-5, freqs.to(DEV), ctx, ctx.groups["g"], lat, rot, across)
     _close(c_q, P.rms_norm(down.double()[:, :Q], qw.double(), 1e-5), tol)
     stored = torch.cat([lat[3, 12:], lat[1, :5]])
     _close(stored, P.rms_norm(down.double()[:, Q:Q + R], kw.double(), 1e-5), tol)
     turned = P.rotate_pairs(down.double()[:, Q + R:], torch.arange(12, 21), 50.0, 2 * pairs)
     _close(torch.cat([rot[3, 12:], rot[1, :5]]), turned, tol)
     assert float(lat[[0, 2, 4]].abs().max()) == 0 and float(lat[1, 5:].abs().max()) == 0
+    assert torch.equal(across.transpose(1, 2), lat)          # the same latents, a page's tokens side by side
 
 
 def _attention_case(dtype, heads, n, r, R, window, length, run, ps, standout, seed):
@@ -183,7 +185,7 @@ def _attention_case(dtype, heads, n, r, R, window, length, run, ps, standout, se
     if standout is not None:
         direction = torch.nn.functional.normalize(torch.randn(R, generator=g), dim=0)
         c[standout] = (direction * 6).to(dtype)
-        q_lat[-1] = (direction * 8).to(dtype)
+        q_lat[-1] = (direction * 20).to(dtype)
     blocks = -(-length // ps)
     order = torch.randperm(blocks + 3, generator=g)[:blocks].tolist()
     lat = torch.randn(blocks + 3, ps, R, generator=g).to(dtype).to(DEV) * 50          # what others left in the pages
@@ -191,16 +193,16 @@ def _attention_case(dtype, heads, n, r, R, window, length, run, ps, standout, se
     for j in range(length):
         lat[order[j // ps], j % ps] = c[j]
         rot[order[j // ps], j % ps] = kr[j]
-    return c, kr, q, q_lat, lat, rot, order
+    return c, kr, q, q_lat, lat, rot, order, lat.transpose(1, 2).contiguous()
 
 
 def _plain_attention(c, kr, q, q_lat, n, window, first, freqs_base, dims, scale):
-    """The mechanism restated: scores q_lat . c + scale * turn(q_r) . k_r under the window, softmax, sum of c."""
+    """The mechanism restated: scores scale * (q_lat . c + turn(q_r) . k_r) under the window, softmax, sum of c."""
     c, kr, q, q_lat = c.double(), kr.double(), q.double(), q_lat.double()
     run, length = q.shape[0], c.shape[0]
     pos = torch.arange(first, first + run)
-    q_r = P.rotate_pairs(q[..., n:], pos, freqs_base, dims) * scale
-    scores = torch.einsum("ihd,jd->hij", q_lat, c) + torch.einsum("ihd,jd->hij", q_r, kr)
+    q_r = P.rotate_pairs(q[..., n:], pos, freqs_base, dims)
+    scores = (torch.einsum("ihd,jd->hij", q_lat, c) + torch.einsum("ihd,jd->hij", q_r, kr)) * scale
     i, j = pos[:, None], torch.arange(length)[None, :]
     seen = (j <= i) & ((i - j < window) if window else torch.ones_like(j <= i))
     prob = torch.softmax(scores.masked_fill(~seen[None], float("-inf")), dim=-1)
@@ -218,22 +220,40 @@ def _plain_attention(c, kr, q, q_lat, n, window, first, freqs_base, dims, scale)
     dict(heads=1, n=32, r=16, R=64, window=33, length=129, run=2, ps=64, back=32),   # a page border: position 96 = 128 - 32
     dict(heads=4, n=8, r=8, R=300, window=1, length=50, run=3, ps=16, back=0),       # a window of one token
     dict(heads=2, n=8, r=4, R=20, window=300, length=280, run=5, ps=16, back=279),   # a window wider than the request
+    # sizes the matrix unit takes (in bfloat16): latents in 16s, rotated parts in 8s
+    dict(heads=3, n=8, r=8, R=48, window=40, length=300, run=1, ps=16, back=39),
+    dict(heads=3, n=8, r=8, R=48, window=40, length=300, run=1, ps=16, back=40),
+    dict(heads=20, n=16, r=16, R=80, window=0, length=700, run=1, ps=64, back=697),  # 20 heads: two blocks of columns
+    dict(heads=2, n=16, r=24, R=160, window=0, length=700, run=37, ps=16, back=699),
+    dict(heads=5, n=8, r=8, R=16, window=17, length=64, run=64, ps=16, back=16),
+    dict(heads=2, n=32, r=16, R=64, window=33, length=300, run=200, ps=64, back=32),  # several tiles of queries
+    dict(heads=1, n=32, r=64, R=512, window=33, length=129, run=2, ps=64, back=32),
+    dict(heads=17, n=8, r=8, R=272, window=100, length=290, run=1, ps=32, back=99),
 ])
-def test_attention_finds_the_key_that_stands_out(name, dtype, tol, case):
+@pytest.mark.parametrize("matrix_unit", [True, False])
+def test_attention_finds_the_key_that_stands_out(name, dtype, tol, case, matrix_unit):
+    if not matrix_unit and dtype == torch.float32:
+        pytest.skip("float32 has the one kernel")
     ops = _ops(dtype)
+    ops.latent_matrix_unit = matrix_unit
     heads, n, r, R, window, length, run, ps = (case[k] for k in ("heads", "n", "r", "R", "window", "length", "run", "ps"))
     standout = length - 1 - case["back"]
-    c, kr, q, q_lat, lat, rot, order = _attention_case(dtype, heads, n, r, R, window, length, run, ps, standout, 7)
+    c, kr, q, q_lat, lat, rot, order, across = _attention_case(dtype, heads, n, r, R, window, length, run, ps, standout, 7)
     dims, base, scale = r - 2 if r > 2 else r, 321.0, 0.4
+    from transformers_neuronx_amd.kernels.attention_plan import attention_plan
     freqs = (base ** (-2.0 * torch.arange(dims // 2, dtype=torch.float64) / dims)).float().to(DEV)
     want, prob = _plain_attention(c, kr, q, q_lat, n, window, length - run, base, dims, scale)
     visible = not window or case["back"] < window
     if case["back"] > 0 or window == 1:
         assert (float(prob[:, -1, standout].min()) > 0.9) == visible
-    ctx = _ctx([run], [length - run], [0], {"g": [order]}, ps)
+    entries = [StepEntry(0, [0] * run, [])]
+    ctx = build_context(entries, [length - run], [0], {"g": np.asarray([order], dtype=np.int32)}, ps, DEV,
+                        {"attention": attention_plan})
     got = ops.latent_attention(q.reshape(run, -1).to(DEV), q_lat.to(DEV), heads, n, r, R, freqs, scale, ctx,
-                               ctx.groups["g"], lat, rot, window or None)
-    _close(got, want, tol)
+                               ctx.groups["g"], lat, rot, across, window or None)
+    # float32: an angle is position * frequency in float32, which at position 700 is 4e-5 of a turn's radian off
+    # the float64 angle, and the scores here are large
+    _close(got, want, max(tol, 4e-5))
 
 
 # ---------------------------------------------------------------- the engine

@@ -1,7 +1,7 @@
 // Latent attention: a token's keys and values are made from one small cached vector c (R elements) and a
 // rotated key part k_r (r elements) that all heads share. The products with the key and value matrices are
 // moved to the query's side, so the kernels read the cache as it lies:
-//   score(i, j, head) = q_lat[i, head] . c[j] + scale * turn(q_r[i, head]) . k_r[j],   out[i, head] = sum_j p_j c[j].
+//   score(i, j, head) = scale * (q_lat[i, head] . c[j] + turn(q_r[i, head]) . k_r[j]),   out[i, head] = sum_j p_j c[j].
 // Here: the norms of the two latents with the store into pages, a product per head (batched), and attention.
 #include "common.h"
 
@@ -26,7 +26,8 @@ latent_norms_kernel(const float* __restrict__ down, int q_rank, int kv_rank, int
                     const int* __restrict__ positions, const int* __restrict__ token_page,
                     const int* __restrict__ token_offset, void* __restrict__ c_q, int dtype,
                     void* __restrict__ latent_pages, void* __restrict__ rotated_pages, size_t latent_stride,
-                    size_t rotated_stride, int num_pages) {
+                    size_t rotated_stride, int num_pages, void* __restrict__ across_pages, size_t across_stride,
+                    int page_size) {
   __shared__ float scratch[4];
   const int t = blockIdx.x;
   const float* row = down + (size_t)t * (q_rank + kv_rank + rot);
@@ -43,7 +44,12 @@ latent_norms_kernel(const float* __restrict__ down, int q_rank, int kv_rank, int
   for (int i = threadIdx.x; i < kv_rank; i += 256) s += lat[i] * lat[i];
   const float rk = 1.f / sqrtf(block_sum<4>(s, scratch) / (float)kv_rank + eps);
   const size_t at = (size_t)page * latent_stride + (size_t)off * kv_rank;
-  for (int i = threadIdx.x; i < kv_rank; i += 256) store_any(latent_pages, dtype, at + i, lat[i] * rk * kv_w[i]);
+  for (int i = threadIdx.x; i < kv_rank; i += 256) {
+    const float v = lat[i] * rk * kv_w[i];
+    store_any(latent_pages, dtype, at + i, v);
+    // the same latent once more with the page's tokens side by side: what the weighted sum contracts over
+    if (across_pages) store_any(across_pages, dtype, (size_t)page * across_stride + (size_t)i * page_size + off, v);
+  }
   const float* kr = lat + kv_rank;
   const size_t rat = (size_t)page * rotated_stride + (size_t)off * rot;
   for (int i = threadIdx.x; i < rot / 2; i += 256) {
@@ -58,8 +64,8 @@ extern "C" int tnx_latent_norms(const float* down, int q_rank, int kv_rank, int 
                                 const float* kv_w, float eps, const float* freqs, int pairs, const int* positions,
                                 const int* token_page, const int* token_offset, void* c_q, int dtype,
                                 void* latent_pages, void* rotated_pages, long long latent_stride,
-                                long long rotated_stride, int num_pages, int page_size, int tokens,
-                                hipStream_t stream) {
+                                long long rotated_stride, int num_pages, int page_size, void* across_pages,
+                                long long across_stride, int tokens, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && q_rank > 0 && kv_rank >= 0 && rot >= 0 && rot % 2 == 0 && (kv_rank == 0 || 2 * pairs <= rot),
               "latent_norms: bad sizes q=%d kv=%d rot=%d pairs=%d", q_rank, kv_rank, rot, pairs);
   TNX_REQUIRE(kv_rank == 0 || (latent_pages && rotated_pages && kv_w && latent_stride >= (long long)page_size * kv_rank &&
@@ -69,7 +75,8 @@ extern "C" int tnx_latent_norms(const float* down, int q_rank, int kv_rank, int 
   latent_norms_kernel<<<tokens, 256, 0, stream>>>(down, q_rank, kv_rank, kv_rank ? rot : 0, q_w, kv_w, eps, freqs, pairs,
                                                   positions, token_page, token_offset, c_q, dtype, latent_pages,
                                                   rotated_pages, (size_t)latent_stride, (size_t)rotated_stride,
-                                                  num_pages);
+                                                  num_pages, kv_rank ? across_pages : nullptr, (size_t)across_stride,
+                                                  page_size);
   TNX_CHECK_LAUNCH("latent_norms");
   return 0;
 }
@@ -178,7 +185,7 @@ latent_attention_any_kernel(const T* __restrict__ q, const T* __restrict__ q_lat
   const int p = positions[t];
   const int* table = block_table + (size_t)token_request[t] * table_width;
   const T* qrow = q + ((size_t)t * heads + h) * (head_size + rot) + head_size;
-  for (int i = threadIdx.x; i < kv_rank; i += 256) ql[i] = to_f32(q_lat[((size_t)t * heads + h) * kv_rank + i]);
+  for (int i = threadIdx.x; i < kv_rank; i += 256) ql[i] = scale * to_f32(q_lat[((size_t)t * heads + h) * kv_rank + i]);
   for (int i = threadIdx.x; i < rot / 2; i += 256) {
     float a = to_f32(qrow[2 * i]), b = to_f32(qrow[2 * i + 1]);
     if (i < pairs) turn_pair(to_f32(qrow[2 * i]), to_f32(qrow[2 * i + 1]), p, freqs[i], a, b);
@@ -270,5 +277,375 @@ extern "C" int tnx_latent_attention_any(const void* q, int dtype, const void* q_
         page_size, num_pages, (const bf16_t*)latent_pages, (const bf16_t*)rotated_pages, (size_t)latent_stride,
         (size_t)rotated_stride, freqs, pairs, scale, heads, head_size, rot, kv_rank, window);
   TNX_CHECK_LAUNCH("latent_attention_any");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------------ attention, bfloat16
+
+// On the matrix unit (MFMA 16x16x32), for latents of a multiple of 16 elements up to 16 * NDB and a rotated part
+// of a multiple of 8 up to LM_ROT. A key is the row [c | k_r] (its two parts lie in pages of their own); the
+// values are the c once more, kept with a page's tokens side by side (`across`: [pages, R, page_size]), since
+// the weighted sum contracts over tokens. As in the attention kernels of the other designs the transposed
+// scores S^T = K Q^T are computed, so that the accumulators (lane = column, four consecutive keys a register
+// group) are at once the B operand of O^T += C^T P^T. A column is a (query, head): in a prompt's run the 16
+// columns of a block of columns are 16 consecutive queries of one head, in decoding 16 heads of the one query,
+// which read the request's keys once between them. q_r is turned by the query's position as it is loaded;
+// the scale meets the float32 scores.
+#define LM_ROT 64
+
+struct LatentPages {
+  const bf16_t* latent;   // [pages, page_size, R]
+  const bf16_t* rotated;  // [pages, page_size, rot]
+  const bf16_t* across;   // [pages, R, page_size]
+  size_t latent_stride, rotated_stride, across_stride;
+  int page_size, num_pages, kv_rank, rot;
+};
+
+// the query operand of one column: chunk `d0 .. d0 + 7` of [q_lat | turn(q_r)]
+__device__ __forceinline__ bf16x8 latent_query_chunk(const bf16_t* q_lat_row, const bf16_t* q_rot_row, int d0, int kv_rank,
+                                                     int rot, int position, const float* freqs, int pairs) {
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (d0 < kv_rank) return *(const bf16x8*)(q_lat_row + d0);
+  if (d0 >= kv_rank + rot) return zero8;
+  const bf16x8 raw = *(const bf16x8*)(q_rot_row + (d0 - kv_rank));
+  bf16x8 out;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int pair = (d0 - kv_rank) / 2 + j;
+    float a = (float)raw[2 * j], b = (float)raw[2 * j + 1];
+    if (pair < pairs) turn_pair((float)raw[2 * j], (float)raw[2 * j + 1], position, freqs[pair], a, b);
+    out[2 * j] = (bf16_t)a;
+    out[2 * j + 1] = (bf16_t)b;
+  }
+  return out;
+}
+
+// S^T of 64 keys from `tile0` on against QB blocks of 16 columns: s[kb][qb][i] = key tile0 + 16 kb + 4 g + i
+template <int NKS, int QB>
+__device__ __forceinline__ void latent_scores(const LatentPages& pg, const int* tab, int tile0, int last_key, int r, int g,
+                                              const bf16x8 (&qf)[QB][NKS], f32x4 (&s)[4][QB]) {
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    const int key0 = tile0 + 16 * kb;
+    f32x4 a[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) a[qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    int page = -1;
+    if (key0 <= last_key) page = tab[key0 / pg.page_size];
+    if (page >= 0 && page < pg.num_pages) {
+      const int off = key0 % pg.page_size + r;
+      const bf16_t* crow = pg.latent + (size_t)page * pg.latent_stride + (size_t)off * pg.kv_rank;
+      const bf16_t* rrow = pg.rotated + (size_t)page * pg.rotated_stride + (size_t)off * pg.rot;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int d0 = 32 * ks + 8 * g;
+        bf16x8 kf = zero8;
+        if (d0 < pg.kv_rank) kf = *(const bf16x8*)(crow + d0);
+        else if (d0 < pg.kv_rank + pg.rot) kf = *(const bf16x8*)(rrow + (d0 - pg.kv_rank));
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) a[qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qb][ks], a[qb], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) s[kb][qb] = a[qb];
+  }
+}
+
+// the running softmax of one block of columns over a tile's masked scores; leaves the probabilities in `s`
+template <int NDB, int QB>
+__device__ __forceinline__ void latent_softmax(f32x4 (&s)[4][QB], int qb, float& m, float& l, f32x4 (&o)[NDB][QB]) {
+  float mx = -INFINITY;
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[kb][qb][i]);
+  mx = rows_max(mx);
+  const float m_new = fmaxf(m, mx);
+  const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = __expf(m - m_safe);
+  float sum = 0.f;
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = __expf(s[kb][qb][i] - m_safe);
+      s[kb][qb][i] = p;
+      sum += p;
+    }
+  sum = rows_sum(sum);
+  l = l * alpha + sum;
+  m = m_new;
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[db][qb][i] *= alpha;
+}
+
+// O^T += C^T P^T for the tile's 64 keys
+template <int NDB, int QB>
+__device__ __forceinline__ void latent_weighted_sum(const LatentPages& pg, const int* tab, int tile0, int last_key, int total,
+                                                    int r, int g, const f32x4 (&s)[4][QB], f32x4 (&o)[NDB][QB]) {
+  const int ndb = pg.kv_rank / 16;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    if (tile0 + 32 * t > last_key) continue;
+    bf16x8 pb[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pb[qb][j] = (bf16_t)s[2 * t + (j >> 2)][qb][j & 3];
+    const bf16_t* vbase[2];
+    bool vok[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int key0 = tile0 + 32 * t + 16 * b;
+      int page = -1;
+      if (key0 <= last_key) page = tab[key0 / pg.page_size];
+      vok[b] = page >= 0 && page < pg.num_pages;
+      vbase[b] = pg.across + (size_t)(vok[b] ? page : 0) * pg.across_stride + key0 % pg.page_size + 4 * g;
+    }
+    const bool tail = tile0 + 32 * t + 32 > total;   // some keys of this step lie beyond the request
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      if (db >= ndb) continue;
+      const int d = 16 * db + r;
+      bf16x8 vf;
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        bf16x4 v4 = {0, 0, 0, 0};
+        if (vok[b]) v4 = *(const bf16x4*)(vbase[b] + (size_t)d * pg.page_size);
+        if (tail) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (tile0 + 32 * t + 16 * b + 4 * g + i >= total) v4[i] = 0;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vf[4 * b + i] = v4[i];
+      }
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) o[db][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[qb], o[db][qb], 0, 0, 0);
+    }
+  }
+}
+
+// A prompt's run: a block of four waves takes 64 QB consecutive queries of one head, a wave 16 QB of them.
+template <int NDB, int QB>
+__global__ void __launch_bounds__(256)
+latent_attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ q_lat, bf16_t* __restrict__ out,
+                               const int* __restrict__ run_start, const int* __restrict__ cached_lens,
+                               const int* __restrict__ table, int table_width, const int* __restrict__ tile_run,
+                               const int* __restrict__ tile_q0, int tile_tokens, LatentPages pg,
+                               const float* __restrict__ freqs, int pairs, float scale, int heads, int head_size,
+                               int window) {
+  constexpr int NKS = (16 * NDB + LM_ROT) / 32;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int parts = tile_tokens / (64 * QB);       // blocks a tile of the plan is cut into
+  const int h = blockIdx.x % heads;
+  const int part = (blockIdx.x / heads) % parts, tile = blockIdx.x / heads / parts;
+  const int run = tile_run[tile];
+  const int t0 = run_start[run], qlen = run_start[run + 1] - t0, cached = cached_lens[run];
+  const int qw0 = tile_q0[tile] + 64 * QB * part + 16 * QB * wave;
+  if (qw0 >= qlen) return;
+  const int* tab = table + (size_t)run * table_width;
+  const int total = cached + qlen;
+  const int R = pg.kv_rank, rot = pg.rot;
+
+  bf16x8 qf[QB][NKS];
+  int qpos[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    const int qi = qw0 + 16 * qb + r;
+    qpos[qb] = cached + qi;
+    const size_t th = (size_t)(t0 + min(qi, qlen - 1)) * heads + h;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks)
+      qf[qb][ks] = latent_query_chunk(q_lat + th * R, q + th * (head_size + rot) + head_size, 32 * ks + 8 * g, R, rot,
+                                      qpos[qb], freqs, pairs);
+  }
+  const int last_q = cached + min(qw0 + 16 * QB - 1, qlen - 1);
+  const int first_q = cached + qw0;
+  const int lo = window > 0 ? max(0, first_q - window + 1) : 0;
+
+  float m[QB], l[QB];
+  f32x4 o[NDB][QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    m[qb] = -INFINITY;
+    l[qb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) o[db][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+  for (int tile0 = (lo / 64) * 64; tile0 <= last_q; tile0 += 64) {
+    f32x4 s[4][QB];
+    latent_scores<NKS, QB>(pg, tab, tile0, last_q, r, g, qf, s);
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = tile0 + 16 * kb + 4 * g + i;
+          const bool ok = key <= qpos[qb] && (window <= 0 || key > qpos[qb] - window);
+          s[kb][qb][i] = ok ? s[kb][qb][i] * scale : -INFINITY;
+        }
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) latent_softmax<NDB, QB>(s, qb, m[qb], l[qb], o);
+    latent_weighted_sum<NDB, QB>(pg, tab, tile0, last_q, total, r, g, s, o);
+  }
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    const int qi = qw0 + 16 * qb + r;
+    if (qi >= qlen) continue;
+    const float inv = l[qb] > 0.f ? 1.f / l[qb] : 0.f;
+    bf16_t* orow = out + ((size_t)(t0 + qi) * heads + h) * R;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      if (16 * db >= R) continue;
+      bf16x4 v4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[db][qb][i] * inv);
+      *(bf16x4*)(orow + 16 * db + 4 * g) = v4;
+    }
+  }
+}
+
+// Decoding: a block takes 16 heads of one request's query; its four waves take the 64-key tiles in turn and
+// their partial results (maximum, sum, weighted latents, float32) meet in LDS, one wave's at a time.
+template <int NDB>
+__global__ void __launch_bounds__(256)
+latent_attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ q_lat, bf16_t* __restrict__ out,
+                               const int* __restrict__ run_start, const int* __restrict__ cached_lens,
+                               const int* __restrict__ table, int table_width, const int* __restrict__ decode_runs,
+                               LatentPages pg, const float* __restrict__ freqs, int pairs, float scale, int heads,
+                               int head_size, int window) {
+  constexpr int NKS = (16 * NDB + LM_ROT) / 32;
+  extern __shared__ float meet[];           // [R][16] weighted latents, then [16] maxima and [16] sums
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int run = decode_runs[blockIdx.x];
+  const int t = run_start[run], p = cached_lens[run];
+  const int h = 16 * blockIdx.y + r;
+  const int* tab = table + (size_t)run * table_width;
+  const int R = pg.kv_rank, rot = pg.rot;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  bf16x8 qf[1][NKS];
+  {
+    const size_t th = (size_t)t * heads + min(h, heads - 1);
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks)
+      qf[0][ks] = h < heads ? latent_query_chunk(q_lat + th * R, q + th * (head_size + rot) + head_size, 32 * ks + 8 * g, R,
+                                                 rot, p, freqs, pairs)
+                            : zero8;
+  }
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  float m = -INFINITY, l = 0.f;
+  f32x4 o[NDB][1];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) o[db][0] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int tile0 = (lo / 64) * 64 + 64 * wave; tile0 <= p; tile0 += 256) {
+    f32x4 s[4][1];
+    latent_scores<NKS, 1>(pg, tab, tile0, p, r, g, qf, s);
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = tile0 + 16 * kb + 4 * g + i;
+        s[kb][0][i] = (key <= p && key >= lo) ? s[kb][0][i] * scale : -INFINITY;
+      }
+    latent_softmax<NDB, 1>(s, 0, m, l, o);
+    latent_weighted_sum<NDB, 1>(pg, tab, tile0, p, p + 1, r, g, s, o);
+  }
+  float* meet_m = meet + (size_t)R * 16;
+  float* meet_l = meet_m + 16;
+  for (int src = 3; src >= 1; --src) {
+    if (wave == src) {
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+        if (16 * db < R)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) meet[(size_t)(16 * db + 4 * g + i) * 16 + r] = o[db][0][i];
+      if (g == 0) {
+        meet_m[r] = m;
+        meet_l[r] = l;
+      }
+    }
+    __syncthreads();
+    if (wave == src - 1) {
+      const float m_b = meet_m[r], l_b = meet_l[r];
+      const float m_new = fmaxf(m, m_b);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float fa = __expf(m - m_safe), fb = __expf(m_b - m_safe);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+        if (16 * db < R)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            o[db][0][i] = o[db][0][i] * fa + meet[(size_t)(16 * db + 4 * g + i) * 16 + r] * fb;
+      l = l * fa + l_b * fb;
+      m = m_new;
+    }
+    __syncthreads();
+  }
+  if (wave != 0 || h >= heads) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  bf16_t* orow = out + ((size_t)t * heads + h) * R;
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) {
+    if (16 * db >= R) continue;
+    bf16x4 v4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[db][0][i] * inv);
+    *(bf16x4*)(orow + 16 * db + 4 * g) = v4;
+  }
+}
+
+// `tiles` runs of several tokens cut into tiles of `tile_tokens` queries (`tile_run`, `tile_q0`), and `decodes`
+// runs of one token (`decode_runs`); either may be none.
+extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void* out, const int* run_start,
+                                         const int* cached_lens, const int* block_table, int table_width, int page_size,
+                                         int num_pages, const int* tile_run, const int* tile_q0, int tiles,
+                                         int tile_tokens, const int* decode_runs, int decodes, const void* latent_pages,
+                                         const void* rotated_pages, const void* across_pages, long long latent_stride,
+                                         long long rotated_stride, long long across_stride, const float* freqs, int pairs,
+                                         float scale, int heads, int head_size, int rot, int kv_rank, int window,
+                                         hipStream_t stream) {
+  TNX_REQUIRE(kv_rank > 0 && kv_rank % 16 == 0 && kv_rank <= 512, "latent_attention_mfma: a latent of %d elements", kv_rank);
+  TNX_REQUIRE(rot >= 0 && rot % 8 == 0 && rot <= LM_ROT && 2 * pairs <= rot, "latent_attention_mfma: a rotated part of %d", rot);
+  TNX_REQUIRE(page_size > 0 && page_size % 16 == 0 && table_width > 0 && num_pages > 0 && window >= 0 && heads > 0,
+              "latent_attention_mfma: bad page sizes");
+  TNX_REQUIRE(kv_rank % 8 == 0 && (head_size + rot) % 8 == 0 && head_size % 8 == 0,
+              "latent_attention_mfma: query rows of %d + %d elements are not read 16 bytes at a time", head_size, rot);
+  TNX_REQUIRE(tile_tokens == 128 || tiles == 0, "latent_attention_mfma: tiles of %d queries", tile_tokens);
+  TNX_REQUIRE(latent_stride % 8 == 0 && rotated_stride % 8 == 0 && across_stride % 4 == 0,
+              "latent_attention_mfma: pages that are not aligned");
+  LatentPages pg = {(const bf16_t*)latent_pages, (const bf16_t*)rotated_pages, (const bf16_t*)across_pages,
+                    (size_t)latent_stride, (size_t)rotated_stride, (size_t)across_stride, page_size, num_pages, kv_rank, rot};
+#define LM_PROMPT(NDB, QB)                                                                                             \
+  latent_attention_prompt_kernel<NDB, QB><<<tiles * (tile_tokens / (64 * QB)) * heads, 256, 0, stream>>>(              \
+      (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, run_start, cached_lens, block_table, table_width, tile_run, \
+      tile_q0, tile_tokens, pg, freqs, pairs, scale, heads, head_size, window)
+#define LM_DECODE(NDB)                                                                                                  \
+  latent_attention_decode_kernel<NDB><<<dim3(decodes, (heads + 15) / 16), 256, (size_t)(kv_rank * 16 + 32) * 4, stream>>>( \
+      (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, run_start, cached_lens, block_table, table_width,           \
+      decode_runs, pg, freqs, pairs, scale, heads, head_size, window)
+  if (tiles > 0) {
+    if (kv_rank <= 64) LM_PROMPT(4, 2);
+    else if (kv_rank <= 128) LM_PROMPT(8, 2);
+    else if (kv_rank <= 256) LM_PROMPT(16, 1);
+    else LM_PROMPT(32, 1);
+    TNX_CHECK_LAUNCH("latent_attention_prompt");
+  }
+  if (decodes > 0) {
+    if (kv_rank <= 64) LM_DECODE(4);
+    else if (kv_rank <= 128) LM_DECODE(8);
+    else if (kv_rank <= 256) LM_DECODE(16);
+    else LM_DECODE(32);
+    TNX_CHECK_LAUNCH("latent_attention_decode");
+  }
+#undef LM_PROMPT
+#undef LM_DECODE
   return 0;
 }

@@ -94,7 +94,11 @@ _SIGNATURES = {
     "latent": {
         "tnx_latent_norms": [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int,
                              _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_ll, _c_ll,
-                             _c_int, _c_int, _c_int, _c_void_p],
+                             _c_int, _c_int, _c_void_p, _c_ll, _c_int, _c_void_p],
+        "tnx_latent_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                                      _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_void_p,
+                                      _c_void_p, _c_void_p, _c_ll, _c_ll, _c_ll, _c_void_p, _c_int, _c_float, _c_int,
+                                      _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_batched_linear": [_c_void_p, _c_int, _c_ll, _c_ll, _c_void_p, _c_int, _c_void_p, _c_int, _c_float, _c_int,
                                _c_int, _c_int, _c_int, _c_void_p],
         "tnx_latent_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
@@ -1077,7 +1081,13 @@ class HipOps:
                    out.numel(), _stream())
         return out
 
-    def _latent_pages(self, latent_pages, rotated_pages, kv_rank, rot, page_size):
+    def _latent_pages(self, latent_pages, rotated_pages, kv_rank, rot, page_size, across_pages=None):
+        if across_pages is not None:
+            a = across_pages
+            if not a.is_cuda or a.dtype != self.dtype or a.dim() != 3 or tuple(a.shape) != (latent_pages.shape[0], kv_rank, page_size) \
+                    or tuple(a.stride()[1:]) != (page_size, 1) or a.stride(0) < kv_rank * page_size:
+                raise ValueError(f"the latents with a page's tokens side by side are [pages, {kv_rank}, {page_size}] in "
+                                 f"{self.dtype}, got {tuple(a.shape)} {a.dtype} with strides {tuple(a.stride())}")
         for pages, name, last in ((latent_pages, "latent pages", kv_rank), (rotated_pages, "rotated pages", rot)):
             if not pages.is_cuda or pages.dtype != self.dtype:
                 raise TypeError(f"{name} must be {self.dtype} on the GPU, got {pages.dtype} on {pages.device}")
@@ -1090,7 +1100,7 @@ class HipOps:
         return latent_pages.shape[0]
 
     def latent_norms(self, down, q_rank, kv_rank, rot, q_weight, kv_weight, eps, freqs, ctx, view, latent_pages,
-                     rotated_pages):
+                     rotated_pages, across_pages=None):
         """See `ReferenceOps.latent_norms`."""
         t = ctx.num_tokens
         _want(down, "down", torch.float32, (t, q_rank + kv_rank + rot))
@@ -1099,7 +1109,7 @@ class HipOps:
         num_pages = 0
         if kv_rank:
             _want(kv_weight, "key/value latent norm", torch.float32, (kv_rank,))
-            num_pages = self._latent_pages(latent_pages, rotated_pages, kv_rank, rot, view.page_size)
+            num_pages = self._latent_pages(latent_pages, rotated_pages, kv_rank, rot, view.page_size, across_pages)
             _want(view.token_page, "token pages", torch.int32, (t,))
             _want(view.token_offset, "token offsets", torch.int32, (t,))
         c_q = torch.empty(t, q_rank, dtype=self.dtype, device=down.device)
@@ -1107,7 +1117,9 @@ class HipOps:
                    float(eps), _ptr(freqs), freqs.numel(), _ptr(ctx.positions), _ptr(view.token_page),
                    _ptr(view.token_offset), _ptr(c_q), _code(self.dtype), _ptr(latent_pages) if kv_rank else None,
                    _ptr(rotated_pages) if kv_rank else None, latent_pages.stride(0) if kv_rank else 0,
-                   rotated_pages.stride(0) if kv_rank else 0, num_pages, view.page_size, t, _stream())
+                   rotated_pages.stride(0) if kv_rank else 0, num_pages, view.page_size,
+                   _ptr(across_pages) if kv_rank and across_pages is not None else None,
+                   across_pages.stride(0) if kv_rank and across_pages is not None else 0, t, _stream())
         return c_q
 
     def batched_linear(self, x, w, alpha=1.0, out_f32=False):
@@ -1126,18 +1138,42 @@ class HipOps:
                          2.0 * t * heads * n * k))
         return out
 
+    latent_matrix_unit = True      # tests clear it to run the any-sizes kernel in bfloat16 too
+
     def latent_attention(self, q, q_lat, num_heads, head_size, rot, kv_rank, freqs, scale, ctx, view, latent_pages,
-                         rotated_pages, window=None):
-        """See `ReferenceOps.latent_attention`."""
+                         rotated_pages, across_pages=None, window=None):
+        """See `ReferenceOps.latent_attention`. bfloat16 with a latent of a multiple of 16 up to 512 elements, a
+        rotated part of a multiple of 8 up to 64 and head sizes in 8s runs on the matrix unit (and reads
+        `across_pages`); everything else, and float32, on the kernel for any sizes."""
         t = ctx.num_tokens
         _want(q, "q", self.dtype, (t, num_heads * (head_size + rot)))
         _want(q_lat, "q_lat", self.dtype, (t, num_heads, kv_rank))
         _want(freqs, "frequencies", torch.float32)
-        num_pages = self._latent_pages(latent_pages, rotated_pages, kv_rank, rot, view.page_size)
+        num_pages = self._latent_pages(latent_pages, rotated_pages, kv_rank, rot, view.page_size, across_pages)
         _want(view.block_table, "block table", torch.int32, (ctx.num_requests, view.width))
         if ctx.max_total > view.width * view.page_size:
             raise ValueError("a request is longer than its block table")
         out = torch.empty(t, num_heads, kv_rank, dtype=self.dtype, device=q.device)
+        fast = (self.dtype == torch.bfloat16 and self.latent_matrix_unit and across_pages is not None
+                and kv_rank % 16 == 0 and kv_rank <= 512 and rot % 8 == 0 and rot <= 64 and head_size % 8 == 0
+                and "tile_run" in ctx.plan and latent_pages.stride(0) % 8 == 0 and rotated_pages.stride(0) % 8 == 0
+                and across_pages.stride(0) % 4 == 0)
+        if fast:
+            tiles, decodes = ctx.plan["tile_run"].numel(), ctx.plan["decode_runs"].numel()
+            seen = float(np.minimum(ctx.cached_lens_host + ctx.run_lens_host, window or 1 << 30).sum())
+            self._call("latent", "tnx_latent_attention_mfma", _ptr(q), _ptr(q_lat), _ptr(out), _ptr(ctx.run_start),
+                       _ptr(ctx.cached_lens), _ptr(view.block_table), view.width, view.page_size, num_pages,
+                       _ptr(ctx.plan["tile_run"]), _ptr(ctx.plan["tile_start"]), tiles, QUERY_TILE,
+                       _ptr(ctx.plan["decode_runs"]), decodes, _ptr(latent_pages), _ptr(rotated_pages),
+                       _ptr(across_pages), latent_pages.stride(0), rotated_pages.stride(0), across_pages.stride(0),
+                       _ptr(freqs), freqs.numel(), float(scale), num_heads, head_size, rot, kv_rank, int(window or 0),
+                       _stream(),
+                       work=(f"{tiles} tiles {decodes} decodes", seen * (2 * kv_rank + rot) * 2,
+                             2.0 * num_heads * (2 * kv_rank + rot) * float(
+                                 (ctx.run_lens_host * np.minimum(ctx.cached_lens_host + (ctx.run_lens_host + 1) / 2,
+                                                                 window or 1 << 30)).sum()))
+                       if debug.timer() is not None else None)
+            return out
         self._call("latent", "tnx_latent_attention_any", _ptr(q), _code(self.dtype), _ptr(q_lat), _ptr(out),
                    _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
                    num_pages, _ptr(latent_pages), _ptr(rotated_pages), latent_pages.stride(0), rotated_pages.stride(0),

@@ -280,10 +280,11 @@ class ReferenceOps:
         return out
 
     def latent_norms(self, down, q_rank, kv_rank, rot, q_weight, kv_weight, eps, freqs, ctx, view, latent_pages,
-                     rotated_pages):
+                     rotated_pages, across_pages=None):
         """`down` float32 `[T, q_rank + kv_rank + rot]`: the first q_rank elements, scaled to unit root mean
         square and weighted, come back in the compute dtype; the next kv_rank likewise go to the tokens' places
-        in `latent_pages`, the last `rot`, turned by the position, to `rotated_pages` (kv_rank 0: none)."""
+        in `latent_pages` (and, the page's tokens side by side, in `across_pages` `[pages, kv_rank, page_size]`), the
+        last `rot`, turned by the position, to `rotated_pages` (kv_rank 0: none)."""
         x = down.float()
 
         def rms(v, w):
@@ -296,6 +297,8 @@ class ReferenceOps:
                 raise RuntimeError("a token of this step has no page")
             off = pos % view.page_size
             latent_pages[page, off] = rms(x[:, q_rank:q_rank + kv_rank], kv_weight).to(latent_pages.dtype)
+            if across_pages is not None:
+                across_pages[page, :, off] = latent_pages[page, off]
             turned = self._turn(x[:, q_rank + kv_rank:q_rank + kv_rank + rot], pos, freqs)
             rotated_pages[page, off] = turned.to(rotated_pages.dtype)
         return c_q
@@ -306,16 +309,17 @@ class ReferenceOps:
         return (y if out_f32 else y.to(self.dtype)).contiguous()
 
     def latent_attention(self, q, q_lat, num_heads, head_size, rot, kv_rank, freqs, scale, ctx, view, latent_pages,
-                         rotated_pages, window=None):
-        """For every token and head: scores q_lat . c[j] + scale * turn(q_r) . k_r[j] over the cached tokens j
+                         rotated_pages, across_pages=None, window=None):
+        """For every token and head: scores scale * (q_lat . c[j] + turn(q_r) . k_r[j]) over the cached tokens j
         of its request with j <= position (and position - j < window), softmax, and the weighted sum of the
-        c[j]: `[T, H, kv_rank]`. `q` `[T, H * (head_size + rot)]` holds q_r, unturned and unscaled, behind
-        each head's `head_size` elements; `q_lat` `[T, H, kv_rank]` is scaled already."""
+        c[j]: `[T, H, kv_rank]`. `q` `[T, H * (head_size + rot)]` holds q_r, unturned, behind each head's
+        `head_size` elements; `q_lat` is `[T, H, kv_rank]`. `across_pages` hold the c[j] once more, a page's
+        tokens side by side, for kernels that sum from there."""
         t = q.shape[0]
         ps = view.page_size
         out = torch.empty(t, num_heads, kv_rank, dtype=torch.float32, device=q.device)
         q_r = q.view(t, num_heads, head_size + rot)[:, :, head_size:].float()
-        q_r = self._turn(q_r, ctx.positions.long(), freqs) * scale
+        q_r = self._turn(q_r, ctx.positions.long(), freqs)
         starts = ctx.run_start.tolist()
         for r in range(ctx.num_requests):
             s, e = starts[r], starts[r + 1]
@@ -326,7 +330,7 @@ class ReferenceOps:
             pages = view.block_table[r, :nb].long().clamp(min=0)
             c = latent_pages[pages].float().reshape(nb * ps, kv_rank)[:total]
             k_r = rotated_pages[pages].float().reshape(nb * ps, rot)[:total]
-            scores = torch.einsum("ihd,jd->hij", q_lat[s:e].float(), c) + torch.einsum("ihd,jd->hij", q_r[s:e], k_r)
+            scores = (torch.einsum("ihd,jd->hij", q_lat[s:e].float(), c) + torch.einsum("ihd,jd->hij", q_r[s:e], k_r)) * scale
             pos = ctx.positions[s:e].long().unsqueeze(1)
             j = torch.arange(total, device=q.device).unsqueeze(0)
             allowed = j <= pos

@@ -137,8 +137,10 @@ class LatentAttention(Mixer):
     in float32, then W_o on the heads side by side. `turn` is the `rotation` (a `rotary` position part).
 
     The cache holds c and k_r, in pages of their own shapes. The products with W_uk and W_uv are moved to the
-    query's side, so that a cached token is read as it lies: q_lat = scale * W_uk^T q_n (R elements a head),
-    score = q_lat . c + scale * q_r . k_r, and the weighted sum of the c[j] goes through W_uv afterwards.
+    query's side, so that a cached token is read as it lies: q_lat = W_uk^T q_n (R elements a head),
+    score = scale * (q_lat . c + q_r . k_r), and the weighted sum of the c[j] goes through W_uv afterwards.
+    c is kept twice, the second time with a page's tokens side by side (`across`), as the other designs'
+    values are: the weighted sum contracts over tokens, and the matrix unit wants them next to each other.
 
     `own_kv=False`: no W_dkv; the mixer reads the cache of another call of the run order, whose R, r and
     rotation are its own. `keep`: the tokens the cache keeps (None: all); a cache that is read by mixers of
@@ -169,7 +171,12 @@ class LatentAttention(Mixer):
     def cache_need(self) -> Optional[CacheNeed]:
         keep = self.keep if self.keep is not None else self.window
         return CacheNeed("paged", window=keep,
-                         page_tensors=(("latent", ("page", self.kv_rank)), ("rotated", ("page", self.rot_size))))
+                         page_tensors=(("latent", ("page", self.kv_rank)), ("rotated", ("page", self.rot_size)),
+                                       ("across", (self.kv_rank, "page"))))
+
+    def step_planners(self):
+        from ..kernels.attention_plan import attention_plan
+        return {"attention": attention_plan}
 
     def param_decls(self, prefix: str) -> List[ParamDecl]:
         dq, uq, dkv, uk, uv, o = (prefix + n for n in self.names)
@@ -216,16 +223,16 @@ class LatentAttention(Mixer):
             raise ValueError("a latent-attention mixer with own_kv writes its cache; one without reads another's")
         ops, view = self.ops, ctx.groups[cache.group]
         heads, n, r = self.num_heads, self.head_size, self.rot_size
-        latent, rotated = cache.pages["latent"], cache.pages["rotated"]
+        latent, rotated, across = cache.pages["latent"], cache.pages["rotated"], cache.pages["across"]
         if latent.shape[-1] != self.kv_rank or rotated.shape[-1] != r:
             raise ValueError(f"the cache holds latents of {latent.shape[-1]} + {rotated.shape[-1]} elements, "
                              f"this mixer reads {self.kv_rank} + {r}")
         down = ops.linear(h, self.w_down, None, out_f32=True)
         c_q = ops.latent_norms(down, self.q_rank, self.kv_rank if self.own_kv else 0, r if self.own_kv else 0,
-                               self.q_norm, self.kv_norm, self.eps, self.freqs, ctx, view, latent, rotated)
+                               self.q_norm, self.kv_norm, self.eps, self.freqs, ctx, view, latent, rotated, across)
         q = ops.linear(c_q, self.w_uq, None)
-        q_lat = ops.batched_linear(q.view(-1, heads, n + r)[:, :, :n], self.w_uk_t, alpha=self.scale)
+        q_lat = ops.batched_linear(q.view(-1, heads, n + r)[:, :, :n], self.w_uk_t)
         o_lat = ops.latent_attention(q, q_lat, heads, n, r, self.kv_rank, self.freqs, self.scale, ctx, view,
-                                     latent, rotated, self.window)
+                                     latent, rotated, across, self.window)
         values = ops.batched_linear(o_lat, self.w_uv)
         return ops.linear(values.view(-1, heads * self.value_size), self.w_o, None, residual=residual, out_f32=True)
