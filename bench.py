@@ -47,6 +47,25 @@ PRESETS = {
     "30b": dict(_OPT, hidden_size=7168, num_hidden_layers=48, num_attention_heads=56, ffn_dim=28672, word_embed_proj_dim=7168),
     "66b": dict(_OPT, hidden_size=9216, num_hidden_layers=64, num_attention_heads=72, ffn_dim=36864, word_embed_proj_dim=9216),
 }
+
+
+def ratesun_config(width, heads, ff, vocab, layers, q_rank, window=1024):
+    """config.json contents of a Ratesun model at the sizes of a published layer: heads of 128 + 64 query/key and
+    128 value elements over a latent of 512, every other layer reading the latent of the one before it."""
+    mixer = dict(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=q_rank, mask=dict(size=window),
+                 rot=dict(base=10000.0, dims=64), scale=(128 + 64) ** -0.5)
+    return dict(architecture="Ratesun", vocab=vocab, width=width, norm=dict(eps=1e-5), residual_mult=0.5, logit_scale=1.0,
+                canon=dict(taps=4), embedding=dict(bigram=dict(buckets=99991, mul_prev=1000003, mul_cur=31)),
+                token_side=dict(dim=64), init_std=0.02, max_positions=4096,
+                layers=[dict(type="latent_attention", mixer=dict(mixer, **({"kv_from": i - 1} if i % 2 else {})),
+                             mlp=dict(kind="dense", ff=ff)) for i in range(layers)])
+
+
+# a new design beside the closest one the engine had, at equal sizes: {design: {size: (its config, the other's)}}
+BESIDE = {"ratesun": {
+    "2048 wide": (lambda n: ratesun_config(2048, 16, 8192, 50272, n, 768), "1.3b"),
+    "4096 wide": (lambda n: ratesun_config(4096, 32, 16384, 50272, n, 1536), "6.7b"),
+}}
 PREFILL_TOKENS = 2048
 PEAK_HBM_GBS = 8000.0                      # MI355X, published
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
@@ -246,6 +265,39 @@ class Bench:
         engine.reset()
         return out
 
+    def kernel_table(self, batch, tokens):
+        """Every kernel of a decode step of `batch` requests at the full context and of a prompt step of `tokens`
+        tokens that says what it moves: {step: {kernel and sizes: [launches, microseconds a launch, GB/s,
+        TFLOP/s, its time's share of what the published peaks would need for its bytes and its flops]}}, and
+        each step's microseconds in all (every launch, also those that say nothing)."""
+        from transformers_neuronx_amd.sampling import SamplingParams
+        engine, out = self.engine, {}
+        for step, count, length in ((f"decode_b{batch}", batch, self.context - 5), (f"prefill_{tokens}", 1, tokens)):
+            engine.reset()
+            decode = step.startswith("decode")
+            for i in range(count):
+                engine.add_request(self.prompt(length), SamplingParams(max_new_tokens=4 if decode else 1, do_sample=False,
+                                                                       ignore_eos=True))
+            if decode:
+                while any(not r.decoding for r in engine.requests.values()):
+                    engine.step()
+                engine.profile(1)
+            else:
+                engine.profile(1)
+                engine.reset()
+                engine.add_request(self.prompt(length), SamplingParams(max_new_tokens=1, do_sample=False, ignore_eos=True))
+            table, _ = engine.profile(1, work=True)
+            rows = {}
+            for name, (calls, ms, nbytes, flops) in sorted(table.items(), key=lambda kv: -kv[1][1]):
+                if nbytes or flops:
+                    need = max(nbytes / (PEAK_HBM_GBS * 1e9), flops / PEAK_FLOPS[self.dtype_name])
+                    rows[name.replace("tnx_", "")] = [calls, round(1e3 * ms / calls, 1), round(nbytes / ms / 1e6),
+                                                      round(flops / ms / 1e9, 1), round(need / (ms * 1e-3), 3)]
+            rows["all launches, us"] = round(1e3 * sum(row[1] for row in table.values()), 1)
+            out[step] = rows
+        engine.reset()
+        return out
+
     def mix(self, requests=64, new_tokens=256):
         """Every request is there at the start; the scheduler mixes portions of prompts with decoding. The
         workload runs twice with other tokens and the second run is timed: the first loads the vendor
@@ -347,7 +399,13 @@ def main():
                     help="time the vendor library's candidates for the many-rows products too")
     ap.add_argument("--big-batch", type=int, default=None,
                     help="the larger batch of `points` (64; cut to what fits the device at the full context)")
+    ap.add_argument("--beside", default=None, choices=sorted(BESIDE),
+                    help="instead: this design at sizes of published layers beside the closest design the engine had, "
+                         "at equal sizes (--layers of them, 4 by default): decode and prompt throughput and every "
+                         "kernel's rates; prints its own line")
     args = ap.parse_args()
+    if args.beside:
+        return beside(args)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
         return 2
@@ -460,6 +518,40 @@ def main():
                 out["kernels"] = {"error": f"{type(e).__name__}: {e}"[:200]}
         if not args.no_extras and args.dtype == "bf16":
             extras(out, bench, raw, args, context)
+    print(json.dumps(out))
+    return 0
+
+
+def beside(args):
+    """`--beside`: for each size, the new design and the other at equal width, heads, inner size, vocabulary and
+    depth, through the same engine: decoding at `--batch` requests and a context of 2,048, a prompt of 2,048
+    tokens in one step, and the table of their kernels."""
+    import torch
+    layers = args.layers or 4
+    context, tokens = args.context or 2048, min(args.prefill_tokens, args.context or 2048)
+    out = {"metric": f"{args.beside} beside OPT at equal sizes: decode tok/s @ batch {args.batch}, prefill tok/s @ {tokens:,} tokens",
+           "unit": "tokens/s", "dtype": args.dtype, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "data": "synthetic (seeded random weights and token ids)", "layers": layers, "context": context, "sizes": {}}
+    for size, (make, preset) in BESIDE[args.beside].items():
+        row = {}
+        for design, raw in ((args.beside, make(layers)), ("opt", dict(PRESETS[preset], num_hidden_layers=layers,
+                                                                        max_position_embeddings=max(2048, context)))):
+            bench = Bench(raw, args.dtype, args.batch, context, step_tokens=tokens)
+            keep_busy(bench.runner.ops, torch, 1.0)
+            value, sec, read = bench.decode(args.batch, args.steps, args.warmup)
+            sec_p, flops = bench.prefill(tokens)
+            row[design] = {"decode_tok_s": round(value, 1), "decode_ms": round(sec * 1e3, 4),
+                           "decode_hbm_frac": round(read / sec / 1e9 / PEAK_HBM_GBS, 4),
+                           "prefill_tok_s": round(tokens / sec_p, 1), "prefill_ms": round(sec_p * 1e3, 3),
+                           "prefill_flops_frac": round(flops / sec_p / PEAK_FLOPS[args.dtype], 4),
+                           "weights_gb": round(bench.model.weight_bytes / 1e9, 3)}
+            log(f"{size} {design}: {row[design]}")
+            if args.dtype == "bf16" and not args.no_points:
+                row[design]["kernels"] = bench.kernel_table(args.batch, tokens)
+            bench.close()
+        out["sizes"][size] = row
+    first = next(iter(out["sizes"].values()))[args.beside]
+    out["value"] = first["decode_tok_s"]
     print(json.dumps(out))
     return 0
 

@@ -134,12 +134,57 @@ batched_linear_kernel(const TX* __restrict__ x, size_t x_row, size_t x_head, con
   }
 }
 
+// The same for few tokens in bfloat16, on the matrix unit: a wave takes one head and 16 of its outputs and makes
+// out^T[n][t] = W[n][:] . x[t][:] for 16 tokens at a time (MFMA 16x16x32: the matrix's rows are the A operand,
+// 16 bytes a lane as they lie, the tokens the B operand). The matrix is read once for every 16 tokens.
+__global__ void __launch_bounds__(256)
+batched_linear_few_kernel(const bf16_t* __restrict__ x, size_t x_row, size_t x_head, const bf16_t* __restrict__ w,
+                          bf16_t* __restrict__ out, float alpha, int tokens, int heads, int n_out, int k_in) {
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int n_blocks = (n_out + 15) / 16;
+  const int id = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (id >= heads * n_blocks) return;
+  const int h = id / n_blocks, nb = id % n_blocks;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int n = 16 * nb + r;
+  const bf16_t* wrow = w + ((size_t)h * n_out + min(n, n_out - 1)) * k_in;
+  for (int t0 = 0; t0 < tokens; t0 += 16) {
+    const int t = t0 + r;
+    const bf16_t* xrow = x + (size_t)min(t, tokens - 1) * x_row + (size_t)h * x_head;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < k_in; k0 += 32) {
+      const int d0 = k0 + 8 * g;
+      const bool in = d0 < k_in;
+      const bf16x8 a = (in && n < n_out) ? *(const bf16x8*)(wrow + d0) : zero8;
+      const bf16x8 b = (in && t < tokens) ? *(const bf16x8*)(xrow + d0) : zero8;
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+    }
+    if (t < tokens) {
+      bf16_t* orow = out + ((size_t)t * heads + h) * n_out;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int no = 16 * nb + 4 * g + i;
+        if (no < n_out) orow[no] = (bf16_t)(alpha * acc[i]);
+      }
+    }
+  }
+}
+
 extern "C" int tnx_batched_linear(const void* x, int x_dtype, long long x_row, long long x_head, const void* w,
                                   int w_dtype, void* out, int out_dtype, float alpha, int tokens, int heads, int n_out,
                                   int k_in, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && heads > 0 && n_out > 0 && k_in > 0, "batched_linear: bad sizes");
   TNX_REQUIRE(heads <= 65535 && (tokens + BL_TILE - 1) / BL_TILE <= 65535, "batched_linear: too many heads or tokens");
   if (tokens == 0) return 0;
+  if (x_dtype == TNX_BF16 && w_dtype == TNX_BF16 && out_dtype == TNX_BF16 && tokens <= 64 && k_in % 8 == 0 &&
+      x_row % 8 == 0 && x_head % 8 == 0 && ((size_t)x % 16) == 0 && ((size_t)w % 16) == 0) {
+    const int waves = heads * ((n_out + 15) / 16);
+    batched_linear_few_kernel<<<(waves + 3) / 4, 256, 0, stream>>>((const bf16_t*)x, (size_t)x_row, (size_t)x_head,
+                                                                   (const bf16_t*)w, (bf16_t*)out, alpha, tokens, heads,
+                                                                   n_out, k_in);
+    TNX_CHECK_LAUNCH("batched_linear_few");
+    return 0;
+  }
   const dim3 grid((n_out + BL_TILE - 1) / BL_TILE, (tokens + BL_TILE - 1) / BL_TILE, heads);
 #define BL_LAUNCH(TX, TW, TO)                                                                                      \
   batched_linear_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((const TX*)x, (size_t)x_row, (size_t)x_head,         \
@@ -511,17 +556,24 @@ latent_attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   }
 }
 
-// Decoding: a block takes 16 heads of one request's query; its four waves take the 64-key tiles in turn and
-// their partial results (maximum, sum, weighted latents, float32) meet in LDS, one wave's at a time.
+// Decoding: a block takes 16 heads of one request's query (the 16 columns) and a share of its keys, 64 at a
+// time. Its four waves work on the same tile: each makes the scores of 16 of the keys, the maxima and sums meet
+// in LDS, the probabilities go to LDS as the B operand of the second product, and there each wave owns a
+// quarter of the latent's blocks of 16 elements, over all 64 keys. So a wave holds a quarter of the result, the
+// keys are read once a block, and the second product reads 8 consecutive tokens of `across`, 16 bytes a lane.
+// With `splits` > 1 the partial results (maximum, sum, weighted latents, float32) go to `part` and a second
+// kernel joins them.
 template <int NDB>
 __global__ void __launch_bounds__(256)
 latent_attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ q_lat, bf16_t* __restrict__ out,
                                const int* __restrict__ run_start, const int* __restrict__ cached_lens,
                                const int* __restrict__ table, int table_width, const int* __restrict__ decode_runs,
                                LatentPages pg, const float* __restrict__ freqs, int pairs, float scale, int heads,
-                               int head_size, int window) {
+                               int head_size, int window, float* __restrict__ part, int splits, int tiles_per_split) {
   constexpr int NKS = (16 * NDB + LM_ROT) / 32;
-  extern __shared__ float meet[];           // [R][16] weighted latents, then [16] maxima and [16] sums
+  constexpr int OWN = (NDB + 3) / 4;           // blocks of 16 latent elements a wave owns: wave, wave + 4, ...
+  __shared__ float tile_max[4][16], tile_sum[4][16];
+  __shared__ __attribute__((aligned(16))) bf16_t prob[16][64 + 8];   // [column][key of the tile]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int run = decode_runs[blockIdx.x];
@@ -531,79 +583,159 @@ latent_attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   const int R = pg.kv_rank, rot = pg.rot;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  bf16x8 qf[1][NKS];
+  bf16x8 qf[NKS];
   {
     const size_t th = (size_t)t * heads + min(h, heads - 1);
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks)
-      qf[0][ks] = h < heads ? latent_query_chunk(q_lat + th * R, q + th * (head_size + rot) + head_size, 32 * ks + 8 * g, R,
-                                                 rot, p, freqs, pairs)
-                            : zero8;
+      qf[ks] = h < heads ? latent_query_chunk(q_lat + th * R, q + th * (head_size + rot) + head_size, 32 * ks + 8 * g, R,
+                                              rot, p, freqs, pairs)
+                         : zero8;
   }
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int first = (lo / 64) * 64 + 64 * tiles_per_split * (int)blockIdx.z;
+  const int end = min(p, first + 64 * tiles_per_split - 1);       // the last key this block may read
   float m = -INFINITY, l = 0.f;
-  f32x4 o[NDB][1];
+  f32x4 o[OWN];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) o[db][0] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  for (int tile0 = (lo / 64) * 64 + 64 * wave; tile0 <= p; tile0 += 256) {
-    f32x4 s[4][1];
-    latent_scores<NKS, 1>(pg, tab, tile0, p, r, g, qf, s);
+  for (int j = 0; j < OWN; ++j) o[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int tile0 = first; tile0 <= end; tile0 += 64) {
+    // this wave's 16 keys against the 16 columns
+    const int key0 = tile0 + 16 * wave;
+    f32x4 a = {0.f, 0.f, 0.f, 0.f};
+    int page = -1;
+    if (key0 <= p) page = tab[key0 / pg.page_size];
+    if (page >= 0 && page < pg.num_pages) {
+      const int off = key0 % pg.page_size + r;
+      const bf16_t* crow = pg.latent + (size_t)page * pg.latent_stride + (size_t)off * R;
+      const bf16_t* rrow = pg.rotated + (size_t)page * pg.rotated_stride + (size_t)off * rot;
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = tile0 + 16 * kb + 4 * g + i;
-        s[kb][0][i] = (key <= p && key >= lo) ? s[kb][0][i] * scale : -INFINITY;
-      }
-    latent_softmax<NDB, 1>(s, 0, m, l, o);
-    latent_weighted_sum<NDB, 1>(pg, tab, tile0, p, p + 1, r, g, s, o);
-  }
-  float* meet_m = meet + (size_t)R * 16;
-  float* meet_l = meet_m + 16;
-  for (int src = 3; src >= 1; --src) {
-    if (wave == src) {
-#pragma unroll
-      for (int db = 0; db < NDB; ++db)
-        if (16 * db < R)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) meet[(size_t)(16 * db + 4 * g + i) * 16 + r] = o[db][0][i];
-      if (g == 0) {
-        meet_m[r] = m;
-        meet_l[r] = l;
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int d0 = 32 * ks + 8 * g;
+        bf16x8 kf = zero8;
+        if (d0 < R) kf = *(const bf16x8*)(crow + d0);
+        else if (d0 < R + rot) kf = *(const bf16x8*)(rrow + (d0 - R));
+        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], a, 0, 0, 0);
       }
     }
-    __syncthreads();
-    if (wave == src - 1) {
-      const float m_b = meet_m[r], l_b = meet_l[r];
-      const float m_new = fmaxf(m, m_b);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float fa = __expf(m - m_safe), fb = __expf(m_b - m_safe);
+    float mx = -INFINITY;
 #pragma unroll
-      for (int db = 0; db < NDB; ++db)
-        if (16 * db < R)
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            o[db][0][i] = o[db][0][i] * fa + meet[(size_t)(16 * db + 4 * g + i) * 16 + r] * fb;
-      l = l * fa + l_b * fb;
-      m = m_new;
+    for (int i = 0; i < 4; ++i) {
+      const int key = key0 + 4 * g + i;
+      a[i] = (key <= p && key >= lo && page >= 0) ? a[i] * scale : -INFINITY;
+      mx = fmaxf(mx, a[i]);
     }
+    mx = rows_max(mx);
+    if (g == 0) tile_max[wave][r] = mx;
     __syncthreads();
-  }
-  if (wave != 0 || h >= heads) return;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  bf16_t* orow = out + ((size_t)t * heads + h) * R;
+    const float m_new = fmaxf(m, fmaxf(fmaxf(tile_max[0][r], tile_max[1][r]), fmaxf(tile_max[2][r], tile_max[3][r])));
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __expf(m - m_safe);
+    float sum = 0.f;
+    bf16x4 p4;
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) {
+    for (int i = 0; i < 4; ++i) {
+      const float pr = __expf(a[i] - m_safe);
+      sum += pr;
+      p4[i] = (bf16_t)pr;
+    }
+    sum = rows_sum(sum);
+    *(bf16x4*)&prob[r][16 * wave + 4 * g] = p4;
+    if (g == 0) tile_sum[wave][r] = sum;
+    __syncthreads();
+    l = l * alpha + ((tile_sum[0][r] + tile_sum[1][r]) + (tile_sum[2][r] + tile_sum[3][r]));
+    m = m_new;
+    // the weighted latents of the blocks this wave owns, over the tile's 64 keys
+    bf16x8 pb[2];
+    const bf16_t* vbase[2];
+    bool vok[2];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      pb[s2] = *(const bf16x8*)&prob[r][32 * s2 + 8 * g];
+      const int k0 = tile0 + 32 * s2 + 8 * g;         // this lane's 8 consecutive keys
+      int pgn = -1;
+      if (k0 <= p) pgn = tab[k0 / pg.page_size];
+      vok[s2] = pgn >= 0 && pgn < pg.num_pages;
+      vbase[s2] = pg.across + (size_t)(vok[s2] ? pgn : 0) * pg.across_stride + k0 % pg.page_size;
+    }
+    const bool tail = tile0 + 63 > p;
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) {
+      const int db = wave + 4 * j;
+      if (16 * db >= R) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[j][i] *= alpha;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        bf16x8 vf = zero8;
+        if (vok[s2]) vf = *(const bf16x8*)(vbase[s2] + (size_t)(16 * db + r) * pg.page_size);
+        if (tail) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (tile0 + 32 * s2 + 8 * g + e > p) vf[e] = 0;
+        }
+        o[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[s2], o[j], 0, 0, 0);
+      }
+    }
+    __syncthreads();       // before the next tile's probabilities are written
+  }
+  if (h >= heads) return;
+  if (splits == 1) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16_t* orow = out + ((size_t)t * heads + h) * R;
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) {
+      const int db = wave + 4 * j;
+      if (16 * db >= R) continue;
+      bf16x4 v4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[j][i] * inv);
+      *(bf16x4*)(orow + 16 * db + 4 * g) = v4;
+    }
+    return;
+  }
+  // [decode run][head][split][R + 2]: the weighted latents, then the maximum and the sum
+  float* mine = part + (((size_t)blockIdx.x * heads + h) * splits + blockIdx.z) * (R + 2);
+#pragma unroll
+  for (int j = 0; j < OWN; ++j) {
+    const int db = wave + 4 * j;
     if (16 * db >= R) continue;
-    bf16x4 v4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[db][0][i] * inv);
-    *(bf16x4*)(orow + 16 * db + 4 * g) = v4;
+    *(f32x4*)(mine + 16 * db + 4 * g) = o[j];
+  }
+  if (wave == 0 && g == 0) {
+    mine[R] = m;
+    mine[R + 1] = l;
+  }
+}
+
+// joins the partial results of the splits of one (decode run, head): one block each
+__global__ void __launch_bounds__(256)
+latent_attention_join_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, const int* __restrict__ run_start,
+                             const int* __restrict__ decode_runs, int heads, int kv_rank, int splits) {
+  const int h = blockIdx.y;
+  const int t = run_start[decode_runs[blockIdx.x]];
+  const float* mine = part + ((size_t)blockIdx.x * heads + h) * splits * (kv_rank + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < splits; ++s) m = fmaxf(m, mine[(size_t)s * (kv_rank + 2) + kv_rank]);
+  const float m_safe = m == -INFINITY ? 0.f : m;
+  float l = 0.f;
+  for (int s = 0; s < splits; ++s)
+    l += mine[(size_t)s * (kv_rank + 2) + kv_rank + 1] * __expf(mine[(size_t)s * (kv_rank + 2) + kv_rank] - m_safe);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  for (int d = threadIdx.x; d < kv_rank; d += 256) {
+    float acc = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float f = __expf(mine[(size_t)s * (kv_rank + 2) + kv_rank] - m_safe);
+      if (f > 0.f) acc += mine[(size_t)s * (kv_rank + 2) + d] * f;
+    }
+    out[((size_t)t * heads + h) * kv_rank + d] = (bf16_t)(acc * inv);
   }
 }
 
 // `tiles` runs of several tokens cut into tiles of `tile_tokens` queries (`tile_run`, `tile_q0`), and `decodes`
-// runs of one token (`decode_runs`); either may be none.
+// runs of one token (`decode_runs`); either may be none. The keys of a decoding request are shared out over
+// `splits` blocks of `tiles_per_split` tiles of 64 keys each; beyond one split `part` holds
+// decodes * heads * splits * (kv_rank + 2) floats.
 extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void* out, const int* run_start,
                                          const int* cached_lens, const int* block_table, int table_width, int page_size,
                                          int num_pages, const int* tile_run, const int* tile_q0, int tiles,
@@ -611,7 +743,7 @@ extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void*
                                          const void* rotated_pages, const void* across_pages, long long latent_stride,
                                          long long rotated_stride, long long across_stride, const float* freqs, int pairs,
                                          float scale, int heads, int head_size, int rot, int kv_rank, int window,
-                                         hipStream_t stream) {
+                                         float* part, int splits, int tiles_per_split, hipStream_t stream) {
   TNX_REQUIRE(kv_rank > 0 && kv_rank % 16 == 0 && kv_rank <= 512, "latent_attention_mfma: a latent of %d elements", kv_rank);
   TNX_REQUIRE(rot >= 0 && rot % 8 == 0 && rot <= LM_ROT && 2 * pairs <= rot, "latent_attention_mfma: a rotated part of %d", rot);
   TNX_REQUIRE(page_size > 0 && page_size % 16 == 0 && table_width > 0 && num_pages > 0 && window >= 0 && heads > 0,
@@ -619,7 +751,9 @@ extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void*
   TNX_REQUIRE(kv_rank % 8 == 0 && (head_size + rot) % 8 == 0 && head_size % 8 == 0,
               "latent_attention_mfma: query rows of %d + %d elements are not read 16 bytes at a time", head_size, rot);
   TNX_REQUIRE(tile_tokens == 128 || tiles == 0, "latent_attention_mfma: tiles of %d queries", tile_tokens);
-  TNX_REQUIRE(latent_stride % 8 == 0 && rotated_stride % 8 == 0 && across_stride % 4 == 0,
+  TNX_REQUIRE(decodes == 0 || (splits >= 1 && splits <= 65535 && tiles_per_split >= 1 && (splits == 1 || part)),
+              "latent_attention_mfma: %d splits of %d tiles", splits, tiles_per_split);
+  TNX_REQUIRE(latent_stride % 8 == 0 && rotated_stride % 8 == 0 && across_stride % 8 == 0,
               "latent_attention_mfma: pages that are not aligned");
   LatentPages pg = {(const bf16_t*)latent_pages, (const bf16_t*)rotated_pages, (const bf16_t*)across_pages,
                     (size_t)latent_stride, (size_t)rotated_stride, (size_t)across_stride, page_size, num_pages, kv_rank, rot};
@@ -627,10 +761,10 @@ extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void*
   latent_attention_prompt_kernel<NDB, QB><<<tiles * (tile_tokens / (64 * QB)) * heads, 256, 0, stream>>>(              \
       (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, run_start, cached_lens, block_table, table_width, tile_run, \
       tile_q0, tile_tokens, pg, freqs, pairs, scale, heads, head_size, window)
-#define LM_DECODE(NDB)                                                                                                  \
-  latent_attention_decode_kernel<NDB><<<dim3(decodes, (heads + 15) / 16), 256, (size_t)(kv_rank * 16 + 32) * 4, stream>>>( \
-      (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, run_start, cached_lens, block_table, table_width,           \
-      decode_runs, pg, freqs, pairs, scale, heads, head_size, window)
+#define LM_DECODE(NDB)                                                                                          \
+  latent_attention_decode_kernel<NDB><<<dim3(decodes, (heads + 15) / 16, splits), 256, 0, stream>>>(            \
+      (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, run_start, cached_lens, block_table, table_width,   \
+      decode_runs, pg, freqs, pairs, scale, heads, head_size, window, part, splits, tiles_per_split)
   if (tiles > 0) {
     if (kv_rank <= 64) LM_PROMPT(4, 2);
     else if (kv_rank <= 128) LM_PROMPT(8, 2);
@@ -644,6 +778,11 @@ extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void*
     else if (kv_rank <= 256) LM_DECODE(16);
     else LM_DECODE(32);
     TNX_CHECK_LAUNCH("latent_attention_decode");
+    if (splits > 1) {
+      latent_attention_join_kernel<<<dim3(decodes, heads), 256, 0, stream>>>(part, (bf16_t*)out, run_start, decode_runs,
+                                                                            heads, kv_rank, splits);
+      TNX_CHECK_LAUNCH("latent_attention_join");
+    }
   }
 #undef LM_PROMPT
 #undef LM_DECODE

@@ -98,7 +98,7 @@ _SIGNATURES = {
         "tnx_latent_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                       _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_void_p,
                                       _c_void_p, _c_void_p, _c_ll, _c_ll, _c_ll, _c_void_p, _c_int, _c_float, _c_int,
-                                      _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                      _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
         "tnx_batched_linear": [_c_void_p, _c_int, _c_ll, _c_ll, _c_void_p, _c_int, _c_void_p, _c_int, _c_float, _c_int,
                                _c_int, _c_int, _c_int, _c_void_p],
         "tnx_latent_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
@@ -427,7 +427,8 @@ class HipOps:
         out_f32 = torch.empty_like(x) if (want_f32 or (want_compute and same)) else None
         out_cd = torch.empty(t, width, dtype=dtype, device=x.device) if (want_compute and not same) else None
         self._call("elementwise", "tnx_layernorm", _ptr(x), _ptr(weight), _ptr(bias), float(eps), _ptr(out_f32),
-                   _ptr(out_cd), _code(dtype), t, width, int(bool(center)), _stream())
+                   _ptr(out_cd), _code(dtype), t, width, int(bool(center)), _stream(),
+                   work=(f"{t}x{width}", t * width * (4 + (4 if out_f32 is not None else 0) + (2 if out_cd is not None else 0)), 0.0))
         return (out_f32 if want_f32 else None), ((out_f32 if same else out_cd) if want_compute else None)
 
     # Steps of few rows: a LayerNorm that only a matrix product reads is done by that product (`fold_norm`,
@@ -1015,7 +1016,7 @@ class HipOps:
                    kept_tokens.numel() if kept_tokens is not None else 0, _ptr(table), _ptr(pairs), _code(table.dtype),
                    table.shape[0], buckets, mul_prev, mul_cur, _ptr(ctx.positions), _ptr(ctx.token_request),
                    _ptr(ctx.run_start), _ptr(ctx.slots), _ptr(last_token), _ptr(out), t, table.shape[1],
-                   ctx.num_requests, _stream())
+                   ctx.num_requests, _stream(), work=(f"{t}x{table.shape[1]}", t * table.shape[1] * (4 + 2 * table.element_size()), 0.0))
         return out
 
     def norm_add(self, y, weight, bias, eps, center, residual, mult=1.0, out=None):
@@ -1032,7 +1033,7 @@ class HipOps:
         else:
             _want(out, "out", torch.float32, (t, width))
         self._call("stream", "tnx_norm_add", _ptr(y), _ptr(weight), _ptr(bias), float(eps), int(bool(center)),
-                   _ptr(residual), float(mult), _ptr(out), t, width, _stream())
+                   _ptr(residual), float(mult), _ptr(out), t, width, _stream(), work=(f"{t}x{width}", t * width * 12, 0.0))
         return out
 
     def input_conv(self, h, weight, state, which, ctx, dtype):
@@ -1049,7 +1050,8 @@ class HipOps:
             mine, stride = state.data_ptr() + which * taps * width * 4, state.stride(0)
         out = torch.empty(t, width, dtype=dtype, device=h.device)
         self._call("stream", "tnx_input_conv", _ptr(h), _ptr(weight), mine, stride, taps, _ptr(ctx.positions),
-                   _ptr(ctx.token_request), _ptr(ctx.run_start), _ptr(ctx.slots), _ptr(out), _code(dtype), t, width, ctx.num_requests, _stream())
+                   _ptr(ctx.token_request), _ptr(ctx.run_start), _ptr(ctx.slots), _ptr(out), _code(dtype), t, width, ctx.num_requests, _stream(),
+                   work=(f"{t}x{width}", t * width * (4 + out.element_size()), 0.0))
         return out
 
     def poly_norm(self, z, coeffs, eps):
@@ -1058,7 +1060,7 @@ class HipOps:
         _want(coeffs, "coefficients", torch.float32, (4,))
         out = torch.empty(z.shape, dtype=self.dtype, device=z.device)
         self._call("stream", "tnx_poly_norm", _ptr(z), _ptr(coeffs), float(eps), _ptr(out), _code(self.dtype),
-                   z.shape[0], z.shape[1], _stream())
+                   z.shape[0], z.shape[1], _stream(), work=(f"{z.shape[0]}x{z.shape[1]}", z.numel() * (4 + out.element_size()), 0.0))
         return out
 
     def mul_columns(self, g, rows, offset):
@@ -1078,7 +1080,7 @@ class HipOps:
             raise ValueError(f"weighted_sum of {count} slots: {history.shape[0]} are there, {weights.numel()} weights")
         out = torch.empty_like(history[0])
         self._call("stream", "tnx_weighted_sum", _ptr(history), _ptr(weights), count, history.stride(0), _ptr(out),
-                   out.numel(), _stream())
+                   out.numel(), _stream(), work=(f"{count}x{out.numel()}", (count + 1) * out.numel() * 4, 0.0))
         return out
 
     def _latent_pages(self, latent_pages, rotated_pages, kv_rank, rot, page_size, across_pages=None):
@@ -1119,8 +1121,11 @@ class HipOps:
                    _ptr(rotated_pages) if kv_rank else None, latent_pages.stride(0) if kv_rank else 0,
                    rotated_pages.stride(0) if kv_rank else 0, num_pages, view.page_size,
                    _ptr(across_pages) if kv_rank and across_pages is not None else None,
-                   across_pages.stride(0) if kv_rank and across_pages is not None else 0, t, _stream())
+                   across_pages.stride(0) if kv_rank and across_pages is not None else 0, t, _stream(),
+                   work=(f"{t}x{q_rank}+{kv_rank}+{rot}", t * ((q_rank + kv_rank + rot) * 4 + (q_rank + 2 * kv_rank + rot) * 2), 0.0))
         return c_q
+
+    batched_library_rows = 64      # from this many rows on a bfloat16 product per head goes to the vendor library (0: never)
 
     def batched_linear(self, x, w, alpha=1.0, out_f32=False):
         """`out[t, h, :] = alpha * w[h] x[t, h, :]`: x `[T, H, K]` (a view whose last axis is dense), w `[H, N, K]`."""
@@ -1131,6 +1136,16 @@ class HipOps:
         _want(w, "w")
         t, heads, k = x.shape
         n = w.shape[1]
+        if (self.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and not out_f32
+                and alpha == 1.0 and t >= self.batched_library_rows > 0):
+            # many rows: the vendor library's batched product, as the plain products of many rows go to it
+            timer = debug.timer()
+            end = timer.start(f"library batched product {t}x{heads}x{n}x{k}", heads * n * k * 2 + t * heads * (k + n) * 2,
+                              2.0 * t * heads * n * k) if timer is not None else None
+            out = torch.bmm(x.transpose(0, 1), w.transpose(1, 2)).transpose(0, 1).contiguous()
+            if end is not None:
+                end.record()
+            return out
         out = torch.empty(t, heads, n, dtype=torch.float32 if out_f32 else self.dtype, device=x.device)
         self._call("latent", "tnx_batched_linear", _ptr(x), _code(x.dtype), x.stride(0), x.stride(1), _ptr(w),
                    _code(w.dtype), _ptr(out), _code(out.dtype), float(alpha), t, heads, n, k, _stream(),
@@ -1157,9 +1172,24 @@ class HipOps:
         fast = (self.dtype == torch.bfloat16 and self.latent_matrix_unit and across_pages is not None
                 and kv_rank % 16 == 0 and kv_rank <= 512 and rot % 8 == 0 and rot <= 64 and head_size % 8 == 0
                 and "tile_run" in ctx.plan and latent_pages.stride(0) % 8 == 0 and rotated_pages.stride(0) % 8 == 0
-                and across_pages.stride(0) % 4 == 0)
+                and across_pages.stride(0) % 8 == 0)
         if fast:
             tiles, decodes = ctx.plan["tile_run"].numel(), ctx.plan["decode_runs"].numel()
+            part, splits, per_split = None, 1, 1
+            if decodes:
+                # The keys of the decoding requests are shared out over blocks until there is about one a compute
+                # unit: a block is 16 heads of a request. A recorded step is sized for the longest request there
+                # can be (a window bounds what any request reads).
+                longest = ctx.length_bound if ctx.length_bound is not None else ctx.plan_host["longest_decode"]
+                key_tiles = (longest - 1) // 64 + 1
+                if window:
+                    key_tiles = min(key_tiles, (window - 1) // 64 + 2)
+                blocks = decodes * -(-num_heads // 16)
+                splits = max(1, min(key_tiles, self.compute_units // blocks, 32))
+                per_split = -(-key_tiles // splits)
+                splits = -(-key_tiles // per_split)
+                if splits > 1:
+                    part = torch.empty(decodes * num_heads * splits * (kv_rank + 2), dtype=torch.float32, device=q.device)
             seen = float(np.minimum(ctx.cached_lens_host + ctx.run_lens_host, window or 1 << 30).sum())
             self._call("latent", "tnx_latent_attention_mfma", _ptr(q), _ptr(q_lat), _ptr(out), _ptr(ctx.run_start),
                        _ptr(ctx.cached_lens), _ptr(view.block_table), view.width, view.page_size, num_pages,
@@ -1167,7 +1197,7 @@ class HipOps:
                        _ptr(ctx.plan["decode_runs"]), decodes, _ptr(latent_pages), _ptr(rotated_pages),
                        _ptr(across_pages), latent_pages.stride(0), rotated_pages.stride(0), across_pages.stride(0),
                        _ptr(freqs), freqs.numel(), float(scale), num_heads, head_size, rot, kv_rank, int(window or 0),
-                       _stream(),
+                       _ptr(part), splits, per_split, _stream(),
                        work=(f"{tiles} tiles {decodes} decodes", seen * (2 * kv_rank + rot) * 2,
                              2.0 * num_heads * (2 * kv_rank + rot) * float(
                                  (ctx.run_lens_host * np.minimum(ctx.cached_lens_host + (ctx.run_lens_host + 1) / 2,
