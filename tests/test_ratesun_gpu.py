@@ -126,12 +126,63 @@ def test_input_convolution_across_steps_of_any_length(name, dtype, tol, taps):
 
 
 @pytest.mark.parametrize("name,dtype,tol", DTYPES)
+@pytest.mark.parametrize("taps,width,joined", [(1, 64, True), (2, 72, False), (3, 2052, True), (4, 128, True), (5, 70, True),
+                                               (4, 4100, False)])
+def test_norm_and_convolution_in_one_launch(name, dtype, tol, taps, width, joined):
+    """The part before joins the stream, the norm and the convolution follow, across steps cut anywhere; widths
+    that the one-launch kernel takes and one that it does not."""
+    ops = _ops(dtype)
+    g = torch.Generator().manual_seed(6)
+    w = torch.randn(width, taps, generator=g)
+    pre_w, pre_b, post_w = torch.randn(width, generator=g), torch.randn(width, generator=g), torch.randn(width, generator=g)
+    lens = {0: 23, 1: 6}
+    x = {k: torch.randn(n, width, generator=g) for k, n in lens.items()}
+    y = {k: torch.randn(n, width, generator=g) * 3 for k, n in lens.items()}
+    want_x = {k: (x[k].double() + 0.3 * P.rms_norm(y[k].double(), post_w.double(), 1e-5)) if joined else x[k].double() for k in x}
+    want = {k: P.input_conv(P.layer_norm(want_x[k], pre_w.double(), pre_b.double(), 1e-5), w.double()) for k in x}
+    state = torch.full((3, 2, taps, width), 7.0, device=DEV) if taps > 1 else None
+    if state is not None:
+        state[1:].zero_()
+    cuts0, cuts1 = [0, 1, 2, 4, 8, 9, 23], [None, None, 0, 5, 6]
+    for s_ in range(len(cuts0) - 1):
+        step = [(0, cuts0[s_], cuts0[s_ + 1], 1)]
+        if s_ + 1 < len(cuts1) and cuts1[s_] is not None:
+            step.append((1, cuts1[s_], cuts1[s_ + 1], 2))
+        xs = torch.cat([x[r][a:b] for r, a, b, _ in step]).to(DEV)
+        ys = torch.cat([y[r][a:b] for r, a, b, _ in step]).to(DEV)
+        ctx = _ctx([b - a for _, a, b, _ in step], [a for _, a, _, _ in step], [slot for _, _, _, slot in step])
+        join = (ys, post_w.to(DEV), None, False, 0.3) if joined else None
+        got_x, out = ops.join_norm_conv(xs, join, (pre_w.to(DEV), pre_b.to(DEV), True, 1e-5), w.to(DEV), state, 0, ctx, dtype)
+        if all(b - a == 1 for _, a, b, _ in step):          # run again, as a recorded step is: the same
+            _, again = ops.join_norm_conv(xs, join, (pre_w.to(DEV), pre_b.to(DEV), True, 1e-5), w.to(DEV), state, 0, ctx, dtype)
+            assert torch.equal(out, again)
+        at = 0
+        for r, a, b, _ in step:
+            _close(out[at:at + b - a], want[r][a:b], max(tol, 3e-6))
+            _close(got_x[at:at + b - a], want_x[r][a:b], 3e-6)
+            at += b - a
+    if state is not None:
+        assert float(state[0].min()) == 7.0 and float(state[1, 1].abs().max()) == 0.0
+
+
+def test_norm_that_joins_leaves_a_copy_for_the_next_product():
+    ops = _ops(torch.bfloat16)
+    g = torch.Generator().manual_seed(1)
+    for width in (64, 1028, 4096, 30):
+        y, x, w = torch.randn(5, width, generator=g), torch.randn(5, width, generator=g), torch.randn(width, generator=g)
+        out, copy = ops.norm_add(y.to(DEV), w.to(DEV), None, 1e-5, False, x.to(DEV), 0.5, None, want_compute=True)
+        _close(out, x.double() + 0.5 * P.rms_norm(y.double(), w.double(), 1e-5), 3e-6)
+        assert copy.dtype == torch.bfloat16 and torch.equal(copy, out.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("name,dtype,tol", DTYPES)
 def test_normed_powers_columns_and_the_average_over_depth(name, dtype, tol):
     ops = _ops(dtype)
     g = torch.Generator().manual_seed(3)
-    z = torch.randn(5, 333, generator=g) * 2
     coeffs = torch.tensor([0.7, -1.3, 0.4, 0.25])
-    _close(ops.poly_norm(z.to(DEV), coeffs.to(DEV), 1e-5), P.poly_norm(z.double(), coeffs.double(), 1e-5), tol)
+    for inner in (333, 320, 5000, 16384, 16388):
+        z = torch.randn(5, inner, generator=g) * 2
+        _close(ops.poly_norm(z.to(DEV), coeffs.to(DEV), 1e-5), P.poly_norm(z.double(), coeffs.double(), 1e-5), tol)
     gate, rows = torch.randn(5, 6, generator=g).to(dtype), torch.randn(5, 30, generator=g).to(dtype)
     _close(ops.mul_columns(gate.to(DEV), rows.to(DEV), 18), gate.double() * rows.double()[:, 18:24], tol)
     hist = torch.randn(6, 5, 77, generator=g)

@@ -96,13 +96,250 @@ norm_add_kernel(const float* __restrict__ y, const float* __restrict__ weight, c
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------ rows in registers
+
+__global__ void conv_state_kernel(const float* __restrict__ h, float* __restrict__ state, size_t slot_stride, int taps,
+                                  const int* __restrict__ positions, const int* __restrict__ run_start,
+                                  const int* __restrict__ slots, int width);
+
+// The same row kernels for widths that are multiples of 4 up to 1024 * PER: a thread holds PER chunks of four
+// floats of the row (chunk c at element 4 * (threadIdx.x + 256 * c)), so a row is read once.
+typedef __attribute__((ext_vector_type(4))) float rf4;
+typedef __attribute__((ext_vector_type(4))) __bf16 rb4;
+
+template <int PER>
+__device__ __forceinline__ void row_load(const float* row, int w4, rf4 (&v)[PER]) {
+#pragma unroll
+  for (int c = 0; c < PER; ++c) {
+    const int i = threadIdx.x + 256 * c;
+    v[c] = i < w4 ? ((const rf4*)row)[i] : (rf4){0.f, 0.f, 0.f, 0.f};
+  }
+}
+
+// v <- (v - mean) * rstd * weight + bias (the mean taken as 0 without `center`), statistics over the block
+template <int PER>
+__device__ __forceinline__ void row_norm(rf4 (&v)[PER], int w4, int width, const float* weight, const float* bias,
+                                         float eps, int center, float* scratch) {
+  float s = 0.f;
+  if (center) {
+#pragma unroll
+    for (int c = 0; c < PER; ++c) s += (v[c].x + v[c].y) + (v[c].z + v[c].w);
+  }
+  const float mean = center ? block_sum<4>(s, scratch) / (float)width : 0.f;
+  float q = 0.f;
+#pragma unroll
+  for (int c = 0; c < PER; ++c) {
+    if (threadIdx.x + 256 * c < w4) {
+      const rf4 d = v[c] - mean;
+      q += (d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w);
+    }
+  }
+  const float rstd = 1.f / sqrtf(block_sum<4>(q, scratch) / (float)width + eps);
+#pragma unroll
+  for (int c = 0; c < PER; ++c) {
+    const int i = threadIdx.x + 256 * c;
+    if (i < w4) {
+      rf4 y = (v[c] - mean) * rstd;
+      if (weight) y = y * ((const rf4*)weight)[i];
+      if (bias) y = y + ((const rf4*)bias)[i];
+      v[c] = y;
+    }
+  }
+}
+
+__device__ __forceinline__ void store_chunk(void* out, int dtype, size_t chunk, rf4 y) {
+  if (dtype == TNX_F32) {
+    ((rf4*)out)[chunk] = y;
+  } else {
+    rb4 o;
+    o.x = (bf16_t)y.x; o.y = (bf16_t)y.y; o.z = (bf16_t)y.z; o.w = (bf16_t)y.w;
+    ((rb4*)out)[chunk] = o;
+  }
+}
+
+// out = residual + mult * norm(y), and a copy in another dtype beside it if asked for
+template <int PER>
+__global__ void __launch_bounds__(256)
+norm_add_rows_kernel(const float* __restrict__ y, const float* __restrict__ weight, const float* __restrict__ bias,
+                     float eps, int center, const float* residual, float mult, float* out, void* __restrict__ copy,
+                     int copy_dtype, int width) {
+  __shared__ float scratch[4];
+  const int w4 = width >> 2;
+  const size_t base = (size_t)blockIdx.x * w4;
+  rf4 v[PER];
+  row_load<PER>(y + (size_t)blockIdx.x * width, w4, v);
+  row_norm<PER>(v, w4, width, weight, bias, eps, center, scratch);
+#pragma unroll
+  for (int c = 0; c < PER; ++c) {
+    const int i = threadIdx.x + 256 * c;
+    if (i < w4) {
+      const rf4 r = ((const rf4*)residual)[base + i] + mult * v[c];
+      ((rf4*)out)[base + i] = r;
+      if (copy) store_chunk(copy, copy_dtype, base + i, r);
+    }
+  }
+}
+
+// What a part reads, in one launch: for a token t of a run, h_t = pre_norm(x'_t), out_t = h_t + conv(h)_t, where
+// x' = x, or with `y`, x' = x + mult * post_norm(y) (the part before, joined to the stream here; x'_t is written
+// to `x_out`). The rows of the taps - 1 tokens before t are made again by this block where they lie in the
+// step's run, and come from the request's state otherwise (`[taps, width]`, position p at place p mod taps).
+// `h_keep`: where a run's last taps - 1 tokens leave their h for the launch that writes the state afterwards;
+// with `write_state` (every run of the step is one token) this kernel writes the state itself.
+template <int PER>
+__global__ void __launch_bounds__(256)
+join_norm_conv_kernel(const float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ post_w,
+                      const float* __restrict__ post_b, int post_center, float mult, float* __restrict__ x_out,
+                      const float* __restrict__ pre_w, const float* __restrict__ pre_b, int pre_center, float eps,
+                      const float* __restrict__ conv_w, float* state, size_t slot_stride, int taps,
+                      const int* __restrict__ positions, const int* __restrict__ token_request,
+                      const int* __restrict__ run_start, const int* __restrict__ slots, void* __restrict__ out,
+                      int out_dtype, float* __restrict__ h_keep, int write_state, int width) {
+  __shared__ float scratch[4];
+  const int w4 = width >> 2;
+  const int t = blockIdx.x;
+  const int r = token_request[t];
+  const int first = run_start[r], n = run_start[r + 1] - first;
+  const int i = t - first, p = positions[t];
+  float* mine = state ? state + (size_t)slots[r] * slot_stride : nullptr;
+  rf4 acc[PER], v[PER];
+#pragma unroll
+  for (int c = 0; c < PER; ++c) acc[c] = (rf4){0.f, 0.f, 0.f, 0.f};
+  for (int back = taps - 1; back >= 0; --back) {
+    if (back <= i) {
+      const size_t row = (size_t)(t - back) * width;
+      row_load<PER>(x + row, w4, v);
+      if (y) {
+        rf4 u[PER];
+        row_load<PER>(y + row, w4, u);
+        row_norm<PER>(u, w4, width, post_w, post_b, eps, post_center, scratch);
+#pragma unroll
+        for (int c = 0; c < PER; ++c) {
+          v[c] = v[c] + mult * u[c];
+          const int k = threadIdx.x + 256 * c;
+          if (back == 0 && k < w4) ((rf4*)(x_out + row))[k] = v[c];
+        }
+      }
+      row_norm<PER>(v, w4, width, pre_w, pre_b, eps, pre_center, scratch);
+    } else if (back <= p && mine) {
+      row_load<PER>(mine + (size_t)((p - back) % taps) * width, w4, v);
+    } else {
+      continue;      // before the request's start: zeros
+    }
+    const int j = taps - 1 - back;
+#pragma unroll
+    for (int c = 0; c < PER; ++c) {
+      const int k = threadIdx.x + 256 * c;
+      if (k < w4) {
+        const float* cw = conv_w + (size_t)(4 * k) * taps + j;
+        const rf4 wj = {cw[0], cw[taps], cw[2 * taps], cw[3 * taps]};
+        acc[c] = acc[c] + wj * v[c];
+        if (back == 0) acc[c] = acc[c] + v[c];
+      }
+    }
+  }
+  // (v holds h_t now)
+#pragma unroll
+  for (int c = 0; c < PER; ++c) {
+    const int k = threadIdx.x + 256 * c;
+    if (k < w4) {
+      store_chunk(out, out_dtype, (size_t)t * w4 + k, acc[c]);
+      if (taps > 1 && i >= n - (taps - 1)) {
+        if (write_state) ((rf4*)(mine + (size_t)(p % taps) * width))[k] = v[c];
+        else ((rf4*)(h_keep + (size_t)t * width))[k] = v[c];
+      }
+    }
+  }
+}
+
+template <int PER>
+__global__ void __launch_bounds__(256)
+poly_norm_rows_kernel(const float* __restrict__ z, const float* __restrict__ coeffs, float eps, void* __restrict__ out,
+                      int out_dtype, int width) {
+  __shared__ float scratch[4];
+  const int w4 = width >> 2;
+  rf4 v[PER];
+  row_load<PER>(z + (size_t)blockIdx.x * width, w4, v);
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+#pragma unroll
+  for (int c = 0; c < PER; ++c) {
+    const rf4 a = v[c] * v[c], b = a * a, d = b * a;
+    s2 += (a.x + a.y) + (a.z + a.w);
+    s4 += (b.x + b.y) + (b.z + b.w);
+    s6 += (d.x + d.y) + (d.z + d.w);
+  }
+  const float r1 = 1.f / sqrtf(block_sum<4>(s2, scratch) / (float)width + eps);
+  const float r2 = 1.f / sqrtf(block_sum<4>(s4, scratch) / (float)width + eps);
+  const float r3 = 1.f / sqrtf(block_sum<4>(s6, scratch) / (float)width + eps);
+  const float a = coeffs[0] * r1, b = coeffs[1] * r2, c3 = coeffs[2] * r3, e = coeffs[3];
+#pragma unroll
+  for (int c = 0; c < PER; ++c) {
+    const int k = threadIdx.x + 256 * c;
+    if (k < w4) {
+      const rf4 x1 = v[c], x2 = x1 * x1;
+      store_chunk(out, out_dtype, (size_t)blockIdx.x * w4 + k, a * x1 + b * x2 + c3 * (x2 * x1) + e);
+    }
+  }
+}
+
+#define ROWS_DISPATCH(width, LAUNCH)      \
+  if (width <= 1024) { LAUNCH(1); }       \
+  else if (width <= 2048) { LAUNCH(2); }  \
+  else if (width <= 4096) { LAUNCH(4); }  \
+  else if (width <= 8192) { LAUNCH(8); }  \
+  else { LAUNCH(16); }
+
+static inline bool rows_fit(int width) { return width % 4 == 0 && width <= 16384; }
+
+// `copy` (optional): the result once more, in `copy_dtype`; widths that the rows-in-registers kernel takes only.
 extern "C" int tnx_norm_add(const float* y, const float* weight, const float* bias, float eps, int center,
-                            const float* residual, float mult, float* out, int tokens, int width, hipStream_t stream) {
+                            const float* residual, float mult, float* out, void* copy, int copy_dtype, int tokens,
+                            int width, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && width > 0 && eps > 0.f, "norm_add: bad sizes tokens=%d width=%d", tokens, width);
   TNX_REQUIRE(y && residual && out && out != y, "norm_add: the result may not lie where the normed rows do");
+  TNX_REQUIRE(!copy || rows_fit(width), "norm_add: no copy beside a row of %d", width);
   if (tokens == 0) return 0;
-  norm_add_kernel<<<tokens, 256, 0, stream>>>(y, weight, bias, eps, center, residual, mult, out, width);
+  if (rows_fit(width)) {
+#define NA_LAUNCH(PER) \
+  norm_add_rows_kernel<PER><<<tokens, 256, 0, stream>>>(y, weight, bias, eps, center, residual, mult, out, copy, copy_dtype, width)
+    ROWS_DISPATCH(width, NA_LAUNCH)
+#undef NA_LAUNCH
+  } else {
+    norm_add_kernel<<<tokens, 256, 0, stream>>>(y, weight, bias, eps, center, residual, mult, out, width);
+  }
   TNX_CHECK_LAUNCH("norm_add");
+  return 0;
+}
+
+// See `join_norm_conv_kernel`. `h_keep` `[tokens, width]` floats is needed unless every run is one token
+// (`single_runs`); widths that `tnx_rows_fit` takes only.
+extern "C" int tnx_rows_fit(int width) { return rows_fit(width) ? 1 : 0; }
+
+extern "C" int tnx_join_norm_conv(const float* x, const float* y, const float* post_w, const float* post_b,
+                                  int post_center, float mult, float* x_out, const float* pre_w, const float* pre_b,
+                                  int pre_center, float eps, const float* conv_w, float* state, long long slot_stride,
+                                  int taps, const int* positions, const int* token_request, const int* run_start,
+                                  const int* slots, void* out, int out_dtype, float* h_keep, int single_runs, int tokens,
+                                  int width, int runs, hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && rows_fit(width) && taps >= 1 && runs >= 0 && eps > 0.f, "join_norm_conv: bad sizes");
+  TNX_REQUIRE(taps == 1 || state, "join_norm_conv: %d taps need the requests' state", taps);
+  TNX_REQUIRE(taps == 1 || single_runs || h_keep, "join_norm_conv: nowhere to leave the inputs that the state takes");
+  TNX_REQUIRE(!y || (x_out && x_out != x), "join_norm_conv: the joined stream needs a place of its own");
+  if (tokens == 0) return 0;
+#define JN_LAUNCH(PER)                                                                                                \
+  join_norm_conv_kernel<PER><<<tokens, 256, 0, stream>>>(x, y, post_w, post_b, post_center, mult, x_out, pre_w, pre_b, \
+                                                         pre_center, eps, conv_w, taps > 1 ? state : nullptr,          \
+                                                         (size_t)slot_stride, taps, positions, token_request,          \
+                                                         run_start, slots, out, out_dtype, h_keep, single_runs, width)
+  ROWS_DISPATCH(width, JN_LAUNCH)
+#undef JN_LAUNCH
+  TNX_CHECK_LAUNCH("join_norm_conv");
+  if (taps > 1 && !single_runs) {
+    conv_state_kernel<<<dim3((width + 255) / 256, runs), 256, 0, stream>>>(h_keep, state, (size_t)slot_stride, taps,
+                                                                          positions, run_start, slots, width);
+    TNX_CHECK_LAUNCH("conv_state");
+  }
   return 0;
 }
 
@@ -200,7 +437,12 @@ extern "C" int tnx_poly_norm(const float* z, const float* coeffs, float eps, voi
                              int width, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && width > 0 && eps > 0.f, "poly_norm: bad sizes tokens=%d width=%d", tokens, width);
   if (tokens == 0) return 0;
-  poly_norm_kernel<<<tokens, 256, 0, stream>>>(z, coeffs, eps, out, out_dtype, width);
+  if (rows_fit(width)) {
+#define PN_LAUNCH(PER) poly_norm_rows_kernel<PER><<<tokens, 256, 0, stream>>>(z, coeffs, eps, out, out_dtype, width)
+    ROWS_DISPATCH(width, PN_LAUNCH)
+#undef PN_LAUNCH
+  } else
+    poly_norm_kernel<<<tokens, 256, 0, stream>>>(z, coeffs, eps, out, out_dtype, width);
   TNX_CHECK_LAUNCH("poly_norm");
   return 0;
 }

@@ -83,8 +83,13 @@ _SIGNATURES = {
         "tnx_embed_pairs": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_ll, _c_ll,
                             _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                             _c_void_p],
-        "tnx_norm_add": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_float, _c_void_p, _c_int,
-                         _c_int, _c_void_p],
+        "tnx_norm_add": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_float, _c_void_p, _c_void_p,
+                         _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_rows_fit": [_c_int],
+        "tnx_join_norm_conv": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_void_p,
+                               _c_void_p, _c_int, _c_float, _c_void_p, _c_void_p, _c_ll, _c_int, _c_void_p, _c_void_p,
+                               _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                               _c_void_p],
         "tnx_input_conv": [_c_void_p, _c_void_p, _c_void_p, _c_ll, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                            _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_poly_norm": [_c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
@@ -1019,8 +1024,9 @@ class HipOps:
                    ctx.num_requests, _stream(), work=(f"{t}x{table.shape[1]}", t * table.shape[1] * (4 + 2 * table.element_size()), 0.0))
         return out
 
-    def norm_add(self, y, weight, bias, eps, center, residual, mult=1.0, out=None):
-        """float32 `residual + mult * norm(y)`; `center` as in `layernorm`."""
+    def norm_add(self, y, weight, bias, eps, center, residual, mult=1.0, out=None, want_compute=False):
+        """float32 `residual + mult * norm(y)`; `center` as in `layernorm`. With `want_compute` the pair (result,
+        its copy in the compute dtype)."""
         _want(y, "y", torch.float32)
         t, width = y.shape
         _want(residual, "residual", torch.float32, (t, width))
@@ -1032,9 +1038,58 @@ class HipOps:
             out = torch.empty_like(y)
         else:
             _want(out, "out", torch.float32, (t, width))
+        copy = None
+        if want_compute and self.dtype != torch.float32 and self.rows_fit(width):
+            copy = torch.empty(t, width, dtype=self.dtype, device=y.device)
         self._call("stream", "tnx_norm_add", _ptr(y), _ptr(weight), _ptr(bias), float(eps), int(bool(center)),
-                   _ptr(residual), float(mult), _ptr(out), t, width, _stream(), work=(f"{t}x{width}", t * width * 12, 0.0))
-        return out
+                   _ptr(residual), float(mult), _ptr(out), _ptr(copy), _code(self.dtype), t, width, _stream(),
+                   work=(f"{t}x{width}", t * width * (12 + (2 if copy is not None else 0)), 0.0))
+        if not want_compute:
+            return out
+        return out, (copy if copy is not None else self.cast(out, self.dtype))
+
+    @staticmethod
+    def rows_fit(width: int) -> bool:
+        """Whether the kernels that hold a row in registers take this width."""
+        return bool(library("stream").tnx_rows_fit(int(width)))
+
+    def join_norm_conv(self, x, join, pre, conv_w, state, which, ctx, dtype):
+        """What a part reads, in one launch where the width allows: `h = pre_norm(x')`, the result `h + conv(h)`
+        as `input_conv` makes it, with `x' = x`, or for `join` = (y, weight, bias, center, mult),
+        `x' = x + mult * post_norm(y)`. `pre` = (weight, bias, center, eps), one eps for both norms. Returns
+        (x', the result in `dtype`)."""
+        t, width = x.shape
+        taps = conv_w.shape[1]
+        pw, pb, pc, eps = pre
+        if not self.rows_fit(width):
+            if join is not None:
+                x = self.norm_add(join[0], join[1], join[2], eps, join[3], x, join[4])
+            h = self.layernorm(x, pw, pb, eps, torch.float32, True, False, pc)[0]
+            return x, self.input_conv(h, conv_w, state, which, ctx, dtype)
+        _want(x, "x", torch.float32)
+        _want(conv_w, "convolution weights", torch.float32, (width, taps))
+        mine, stride = None, 0
+        if taps > 1:
+            _want(state, "convolution state", torch.float32)
+            if state.dim() != 4 or tuple(state.shape[2:]) != (taps, width) or not 0 <= which < state.shape[1]:
+                raise ValueError(f"convolution state is [slots, parts, {taps}, {width}], got {tuple(state.shape)}")
+            mine, stride = state.data_ptr() + which * taps * width * 4, state.stride(0)
+        y = jw = jb = x_out = None
+        jc, mult = 1, 1.0
+        if join is not None:
+            y, jw, jb, jc, mult = join
+            _want(y, "y", torch.float32, (t, width))
+            x_out = torch.empty_like(x)
+        single = bool(ctx.run_lens_host.max() == 1)
+        keep = torch.empty(t, width, dtype=torch.float32, device=x.device) if taps > 1 and not single else None
+        out = torch.empty(t, width, dtype=dtype, device=x.device)
+        self._call("stream", "tnx_join_norm_conv", _ptr(x), _ptr(y), _ptr(jw), _ptr(jb), int(bool(jc)), float(mult),
+                   _ptr(x_out), _ptr(pw), _ptr(pb), int(bool(pc)), float(eps), _ptr(conv_w), mine, stride, taps,
+                   _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(ctx.run_start), _ptr(ctx.slots), _ptr(out),
+                   _code(dtype), _ptr(keep), int(single), t, width, ctx.num_requests, _stream(),
+                   work=(f"{t}x{width}{' joined' if join is not None else ''}",
+                         t * width * (4 + out.element_size() + (8 if join is not None else 0)), 0.0))
+        return (x_out if join is not None else x), out
 
     def input_conv(self, h, weight, state, which, ctx, dtype):
         """See `ReferenceOps.input_conv`."""

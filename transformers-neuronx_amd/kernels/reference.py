@@ -211,14 +211,25 @@ class ReferenceOps:
         last_token[slots, pos[starts[1:] - 1] & 1] = ids[starts[1:] - 1].to(last_token.dtype)
         return table[ids].float() + pairs[rows].float()
 
-    def norm_add(self, y, weight, bias, eps, center, residual, mult=1.0, out=None):
-        """float32 `residual + mult * norm(y)`; `center` as in `layernorm`."""
+    def norm_add(self, y, weight, bias, eps, center, residual, mult=1.0, out=None, want_compute=False):
+        """float32 `residual + mult * norm(y)`; `center` as in `layernorm`. With `want_compute` the pair (result,
+        its copy in the compute dtype)."""
         normed = self.layernorm(y, weight, bias, eps, torch.float32, True, False, center)[0]
         result = residual.float() + mult * normed
         if out is not None:
             out.copy_(result)
-            return out
-        return result
+            result = out
+        return (result, result.to(self.dtype)) if want_compute else result
+
+    def join_norm_conv(self, x, join, pre, conv_w, state, which, ctx, dtype):
+        """What a part reads: `h = pre_norm(x')`, the result `h + conv(h)` as `input_conv` makes it, with `x' = x`,
+        or for `join` = (y, weight, bias, center, mult), `x' = x + mult * post_norm(y)`. `pre` = (weight, bias,
+        center, eps), one eps for both norms. Returns (x', the result in `dtype`)."""
+        pw, pb, pc, eps = pre
+        if join is not None:
+            x = self.norm_add(join[0], join[1], join[2], eps, join[3], x, join[4])
+        h = self.layernorm(x, pw, pb, eps, torch.float32, True, False, pc)[0]
+        return x, self.input_conv(h, conv_w, state, which, ctx, dtype)
 
     def input_conv(self, h, weight, state, which, ctx, dtype):
         """`h + conv(h)`: conv(h)_t = sum_j weight[:, j] h_(t - taps + 1 + j) over the tokens of t's own request;

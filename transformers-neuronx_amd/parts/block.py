@@ -133,13 +133,23 @@ class SandwichBlock(Block):
     def flops_per_token(self, keys: float = 0.0) -> float:
         return 4.0 * self.side["dim"] * self.width if self.side else 0.0
 
-    def _input(self, norm, x, which, ctx):
-        """What a part reads: the norm of the stream, with the convolution over the request's tokens."""
-        if self.taps <= 0:
-            return norm.forward(x, False, True)[1]
-        h = norm.forward(x, True, False)[0]
+    def _input(self, norm, x, which, ctx, join=None):
+        """What a part reads: the norm of the stream, with the convolution over the request's tokens. `join` =
+        (y, post norm): the part before joins the stream first, x + mult * post_norm(y). Returns (the stream,
+        what the part reads). One launch where both norms can be applied inside a kernel of the backend's."""
         state = ctx.call_state.state["inputs"] if self.taps > 1 else None
-        return self.ops.input_conv(h, self.conv_w[which], state, which, ctx, self.dtype)
+        pre = norm.fused_form() if hasattr(norm, "fused_form") else None
+        post = join[1].fused_form() if join is not None and hasattr(join[1], "fused_form") else None
+        if self.taps > 0 and pre is not None and (join is None or (post is not None and post[3] == pre[3])) \
+                and not debug.tapping():
+            joined = (join[0], post[0], post[1], post[2], self.mult) if join is not None else None
+            return self.ops.join_norm_conv(x, joined, pre, self.conv_w[which], state, which, ctx, self.dtype)
+        if join is not None:
+            x = debug.tap("after_mixer", join[1].add_to(join[0], x, self.mult))
+        if self.taps <= 0:
+            return x, norm.forward(x, False, True)[1]
+        h = norm.forward(x, True, False)[0]
+        return x, self.ops.input_conv(h, self.conv_w[which], state, which, ctx, self.dtype)
 
     def forward(self, stream: Stream, ctx, cache) -> Stream:
         ops = self.ops
@@ -153,21 +163,27 @@ class SandwichBlock(Block):
             raise ValueError(f"the average over depth has {self.depth_slots} places and the run order more calls")
         place = history[filled] if self.depth_average else None       # where this call's own result goes
 
-        h = self._input(self.mixer_norm, x, 0, ctx)
+        x, h = self._input(self.mixer_norm, x, 0, ctx)
         y = self.mixer.forward(h, ctx, cache, None)
-        last = not self.has_ff and not self.side
-        x = debug.tap("after_mixer", self.mixer_post.add_to(y, x, self.mult, place if last else None))
+        compute = None
         if self.has_ff:
-            h = self._input(self.feed_forward_norm, x, 1, ctx)
+            x, h = self._input(self.feed_forward_norm, x, 1, ctx, join=(y, self.mixer_post))
             y = self.feed_forward.forward(h, ctx, None)
-            x = self.ff_post.add_to(y, x, self.mult, place if not self.side else None)
+            if self.side:
+                x, compute = self.ff_post.add_to(y, x, self.mult, None, want_compute=True)
+            else:
+                x = self.ff_post.add_to(y, x, self.mult, place)
+        elif self.side:
+            x, compute = self.mixer_post.add_to(y, x, self.mult, None, want_compute=True)
+        else:
+            x = self.mixer_post.add_to(y, x, self.mult, place)
         if self.side:
             s = self.side
             rows = ctx.memo.get(("table rows", s["table"]))
             if rows is None:        # the tokens' rows, looked up once a step for all layers
                 rows = ctx.memo[("table rows", s["table"])] = ops.embed(ctx.token_ids, self.side_table, self.dtype,
                                                                        ctx.kept_tokens)
-            g = ops.linear(ops.cast(x, self.dtype), self.side_gate, None, act="gelu_new")
+            g = ops.linear(compute, self.side_gate, None, act="gelu_new")
             g = ops.mul_columns(g, rows, s["offset"])
             y = ops.linear(g, self.side_proj, None, out_f32=True)
             x = ops.norm_add(y, self.side_norm, None, s["eps"], False, x, self.mult, place)

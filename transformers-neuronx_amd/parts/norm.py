@@ -35,9 +35,13 @@ class LayerNorm(Norm):
     def forward(self, x, want_f32: bool, want_compute: bool):
         return self.ops.layernorm(x, self.weight, self.bias, self.eps, self.dtype, want_f32, want_compute)
 
-    def add_to(self, y, residual, mult: float = 1.0, out=None):
+    def add_to(self, y, residual, mult: float = 1.0, out=None, want_compute: bool = False):
         """`residual + mult * norm(y)` in float32 (into `out`, if given): the norm that follows a part."""
-        return self.ops.norm_add(y, self.weight, self.bias, self.eps, True, residual, mult, out)
+        return self.ops.norm_add(y, self.weight, self.bias, self.eps, True, residual, mult, out, want_compute)
+
+    def fused_form(self):
+        """(weight, bias, center, eps) for kernels that apply the norm inside a launch of their own."""
+        return self.weight, self.bias, True, self.eps
 
     def fold_into(self, w) -> bool:
         return self.ops.fold_norm(w, self.weight, self.bias)
@@ -66,8 +70,11 @@ class RMSNorm(Norm):
     def forward(self, x, want_f32: bool, want_compute: bool):
         return self.ops.layernorm(x, self.weight, None, self.eps, self.dtype, want_f32, want_compute, center=False)
 
-    def add_to(self, y, residual, mult: float = 1.0, out=None):
-        return self.ops.norm_add(y, self.weight, None, self.eps, False, residual, mult, out)
+    def add_to(self, y, residual, mult: float = 1.0, out=None, want_compute: bool = False):
+        return self.ops.norm_add(y, self.weight, None, self.eps, False, residual, mult, out, want_compute)
+
+    def fused_form(self):
+        return self.weight, None, False, self.eps
 
     def fold_into(self, w) -> bool:
         return self.ops.fold_norm(w, self.weight, None, center=False)
