@@ -235,3 +235,16 @@ def test_generation_through_the_entry_point_on_the_host(tmp_path):
     out = model.sample(ids, sequence_length=14, top_k=1)
     for row in range(2):
         assert out[row, 4:].tolist() == _greedy(cfg, w, ids[row].tolist(), 10)
+
+
+def test_bindings_pass_as_many_arguments_as_the_entry_points_take():
+    """Every C entry point of the package's kernel modules is declared with as many argument types as its source
+    has parameters (a call with one too many would hand the launch a stream cut to 32 bits)."""
+    import re
+    from transformers_neuronx_amd.kernels import build, hip
+    for module in build.MODULES:
+        source = open(os.path.join(build.CSRC, f"{module}.hip")).read()
+        for name, types in hip._SIGNATURES[module].items():
+            found = re.search(r'extern "C" int ' + name + r"\(([^)]*)\)", source)
+            assert found, f"{module}.hip has no entry point {name}"
+            assert len([a for a in found.group(1).split(",") if a.strip()]) == len(types), name

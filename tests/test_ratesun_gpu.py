@@ -281,12 +281,15 @@ def _plain_attention(c, kr, q, q_lat, n, window, first, freqs_base, dims, scale)
     dict(heads=1, n=32, r=64, R=512, window=33, length=129, run=2, ps=64, back=32),
     dict(heads=17, n=8, r=8, R=272, window=100, length=290, run=1, ps=32, back=99),
 ])
-@pytest.mark.parametrize("matrix_unit", [True, False])
-def test_attention_finds_the_key_that_stands_out(name, dtype, tol, case, matrix_unit):
-    if not matrix_unit and dtype == torch.float32:
+@pytest.mark.parametrize("kernel", ["shared", "alone", "any"])
+def test_attention_finds_the_key_that_stands_out(name, dtype, tol, case, kernel):
+    """`kernel`: bfloat16 on the matrix unit with a block's waves sharing a tile, or each walking the keys alone
+    (prompt runs), or the kernel for any sizes, which is also float32's."""
+    if kernel != "any" and dtype == torch.float32:
         pytest.skip("float32 has the one kernel")
     ops = _ops(dtype)
-    ops.latent_matrix_unit = matrix_unit
+    ops.latent_matrix_unit = kernel != "any"
+    ops.latent_prompt_kind = 1 if kernel == "alone" else 0
     heads, n, r, R, window, length, run, ps = (case[k] for k in ("heads", "n", "r", "R", "window", "length", "run", "ps"))
     standout = length - 1 - case["back"]
     c, kr, q, q_lat, lat, rot, order, across = _attention_case(dtype, heads, n, r, R, window, length, run, ps, standout, 7)

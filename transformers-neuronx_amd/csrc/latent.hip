@@ -708,6 +708,177 @@ latent_attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   }
 }
 
+// A prompt's run with the waves of a block on one tile, as in decoding: the columns are 16 consecutive queries
+// of HB heads (HB blocks of 16 columns, which see the same keys), each wave makes the scores of 16 of a tile's 64
+// keys for all of them and owns a quarter of the latent's blocks in the second product. Against a wave that walks
+// the keys alone for its own 16 queries, the keys are read once a block and not once a wave, and every operand
+// that is loaded meets HB products.
+template <int NDB, int HB>
+__global__ void __launch_bounds__(256)
+latent_attention_prompt_shared_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ q_lat,
+                                      bf16_t* __restrict__ out, const int* __restrict__ run_start,
+                                      const int* __restrict__ cached_lens, const int* __restrict__ table,
+                                      int table_width, const int* __restrict__ tile_run,
+                                      const int* __restrict__ tile_q0, int tile_tokens, LatentPages pg,
+                                      const float* __restrict__ freqs, int pairs, float scale, int heads,
+                                      int head_size, int window) {
+  constexpr int NKS = (16 * NDB + LM_ROT) / 32;
+  constexpr int OWN = (NDB + 3) / 4;
+  __shared__ float tile_max[4][HB][16], tile_sum[4][HB][16];
+  __shared__ __attribute__((aligned(16))) bf16_t prob[HB][16][64 + 8];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int head_groups = (heads + HB - 1) / HB, parts = tile_tokens / 16;
+  const int hg = blockIdx.x % head_groups;
+  const int part = (blockIdx.x / head_groups) % parts, tile = blockIdx.x / head_groups / parts;
+  const int run = tile_run[tile];
+  const int t0 = run_start[run], qlen = run_start[run + 1] - t0, cached = cached_lens[run];
+  const int q0 = tile_q0[tile] + 16 * part;
+  if (q0 >= qlen) return;
+  const int* tab = table + (size_t)run * table_width;
+  const int total = cached + qlen;
+  const int R = pg.kv_rank, rot = pg.rot;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int qi = q0 + r, qpos = cached + qi;
+
+  bf16x8 qf[HB][NKS];
+#pragma unroll
+  for (int hb = 0; hb < HB; ++hb) {
+    const int h = HB * hg + hb;
+    const size_t th = (size_t)(t0 + min(qi, qlen - 1)) * heads + min(h, heads - 1);
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks)
+      qf[hb][ks] = h < heads ? latent_query_chunk(q_lat + th * R, q + th * (head_size + rot) + head_size, 32 * ks + 8 * g, R,
+                                                  rot, qpos, freqs, pairs)
+                             : zero8;
+  }
+  const int first_q = cached + q0, last_q = cached + min(q0 + 15, qlen - 1);
+  const int lo = window > 0 ? max(0, first_q - window + 1) : 0;
+  float m[HB], l[HB];
+  f32x4 o[OWN][HB];
+#pragma unroll
+  for (int hb = 0; hb < HB; ++hb) {
+    m[hb] = -INFINITY;
+    l[hb] = 0.f;
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) o[j][hb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+  for (int tile0 = (lo / 64) * 64; tile0 <= last_q; tile0 += 64) {
+    const int key0 = tile0 + 16 * wave;
+    f32x4 a[HB];
+#pragma unroll
+    for (int hb = 0; hb < HB; ++hb) a[hb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    int page = -1;
+    if (key0 <= last_q) page = tab[key0 / pg.page_size];
+    if (page >= 0 && page < pg.num_pages) {
+      const int off = key0 % pg.page_size + r;
+      const bf16_t* crow = pg.latent + (size_t)page * pg.latent_stride + (size_t)off * R;
+      const bf16_t* rrow = pg.rotated + (size_t)page * pg.rotated_stride + (size_t)off * rot;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int d0 = 32 * ks + 8 * g;
+        bf16x8 kf = zero8;
+        if (d0 < R) kf = *(const bf16x8*)(crow + d0);
+        else if (d0 < R + rot) kf = *(const bf16x8*)(rrow + (d0 - R));
+#pragma unroll
+        for (int hb = 0; hb < HB; ++hb) a[hb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[hb][ks], a[hb], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int hb = 0; hb < HB; ++hb) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = key0 + 4 * g + i;
+        const bool ok = page >= 0 && key <= qpos && (window <= 0 || key > qpos - window);
+        a[hb][i] = ok ? a[hb][i] * scale : -INFINITY;
+        mx = fmaxf(mx, a[hb][i]);
+      }
+      mx = rows_max(mx);
+      if (g == 0) tile_max[wave][hb][r] = mx;
+    }
+    __syncthreads();
+    float alpha[HB];
+#pragma unroll
+    for (int hb = 0; hb < HB; ++hb) {
+      const float m_new = fmaxf(m[hb], fmaxf(fmaxf(tile_max[0][hb][r], tile_max[1][hb][r]),
+                                             fmaxf(tile_max[2][hb][r], tile_max[3][hb][r])));
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      alpha[hb] = __expf(m[hb] - m_safe);
+      m[hb] = m_new;
+      float sum = 0.f;
+      bf16x4 p4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pr = __expf(a[hb][i] - m_safe);
+        sum += pr;
+        p4[i] = (bf16_t)pr;
+      }
+      sum = rows_sum(sum);
+      *(bf16x4*)&prob[hb][r][16 * wave + 4 * g] = p4;
+      if (g == 0) tile_sum[wave][hb][r] = sum;
+    }
+    __syncthreads();
+    bf16x8 pb[HB][2];
+#pragma unroll
+    for (int hb = 0; hb < HB; ++hb) {
+      l[hb] = l[hb] * alpha[hb] + ((tile_sum[0][hb][r] + tile_sum[1][hb][r]) + (tile_sum[2][hb][r] + tile_sum[3][hb][r]));
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) pb[hb][s2] = *(const bf16x8*)&prob[hb][r][32 * s2 + 8 * g];
+    }
+    const bf16_t* vbase[2];
+    bool vok[2];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      const int k0 = tile0 + 32 * s2 + 8 * g;
+      int pgn = -1;
+      if (k0 <= last_q) pgn = tab[k0 / pg.page_size];
+      vok[s2] = pgn >= 0 && pgn < pg.num_pages;
+      vbase[s2] = pg.across + (size_t)(vok[s2] ? pgn : 0) * pg.across_stride + k0 % pg.page_size;
+    }
+    const bool tail = tile0 + 64 > total;
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) {
+      const int db = wave + 4 * j;
+      if (16 * db >= R) continue;
+#pragma unroll
+      for (int hb = 0; hb < HB; ++hb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[j][hb][i] *= alpha[hb];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        bf16x8 vf = zero8;
+        if (vok[s2]) vf = *(const bf16x8*)(vbase[s2] + (size_t)(16 * db + r) * pg.page_size);
+        if (tail) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (tile0 + 32 * s2 + 8 * g + e >= total) vf[e] = 0;
+        }
+#pragma unroll
+        for (int hb = 0; hb < HB; ++hb) o[j][hb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[hb][s2], o[j][hb], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+  if (qi >= qlen) return;
+#pragma unroll
+  for (int hb = 0; hb < HB; ++hb) {
+    const int h = HB * hg + hb;
+    if (h >= heads) continue;
+    const float inv = l[hb] > 0.f ? 1.f / l[hb] : 0.f;
+    bf16_t* orow = out + ((size_t)(t0 + qi) * heads + h) * R;
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) {
+      const int db = wave + 4 * j;
+      if (16 * db >= R) continue;
+      bf16x4 v4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[j][hb][i] * inv);
+      *(bf16x4*)(orow + 16 * db + 4 * g) = v4;
+    }
+  }
+}
+
 // joins the partial results of the splits of one (decode run, head): one block each
 __global__ void __launch_bounds__(256)
 latent_attention_join_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, const int* __restrict__ run_start,
@@ -735,7 +906,8 @@ latent_attention_join_kernel(const float* __restrict__ part, bf16_t* __restrict_
 // `tiles` runs of several tokens cut into tiles of `tile_tokens` queries (`tile_run`, `tile_q0`), and `decodes`
 // runs of one token (`decode_runs`); either may be none. The keys of a decoding request are shared out over
 // `splits` blocks of `tiles_per_split` tiles of 64 keys each; beyond one split `part` holds
-// decodes * heads * splits * (kv_rank + 2) floats.
+// decodes * heads * splits * (kv_rank + 2) floats. `prompt_kind` 0: the prompt kernel whose waves share a tile;
+// 1: the one whose waves walk the keys each for its own queries.
 extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void* out, const int* run_start,
                                          const int* cached_lens, const int* block_table, int table_width, int page_size,
                                          int num_pages, const int* tile_run, const int* tile_q0, int tiles,
@@ -743,7 +915,8 @@ extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void*
                                          const void* rotated_pages, const void* across_pages, long long latent_stride,
                                          long long rotated_stride, long long across_stride, const float* freqs, int pairs,
                                          float scale, int heads, int head_size, int rot, int kv_rank, int window,
-                                         float* part, int splits, int tiles_per_split, hipStream_t stream) {
+                                         float* part, int splits, int tiles_per_split, int prompt_kind,
+                                         hipStream_t stream) {
   TNX_REQUIRE(kv_rank > 0 && kv_rank % 16 == 0 && kv_rank <= 512, "latent_attention_mfma: a latent of %d elements", kv_rank);
   TNX_REQUIRE(rot >= 0 && rot % 8 == 0 && rot <= LM_ROT && 2 * pairs <= rot, "latent_attention_mfma: a rotated part of %d", rot);
   TNX_REQUIRE(page_size > 0 && page_size % 16 == 0 && table_width > 0 && num_pages > 0 && window >= 0 && heads > 0,
@@ -765,13 +938,24 @@ extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void*
   latent_attention_decode_kernel<NDB><<<dim3(decodes, (heads + 15) / 16, splits), 256, 0, stream>>>(            \
       (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, run_start, cached_lens, block_table, table_width,   \
       decode_runs, pg, freqs, pairs, scale, heads, head_size, window, part, splits, tiles_per_split)
-  if (tiles > 0) {
+#define LM_SHARED(NDB, HB)                                                                                            \
+  latent_attention_prompt_shared_kernel<NDB, HB><<<tiles * (tile_tokens / 16) * ((heads + HB - 1) / HB), 256, 0, stream>>>( \
+      (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, run_start, cached_lens, block_table, table_width, tile_run,   \
+      tile_q0, tile_tokens, pg, freqs, pairs, scale, heads, head_size, window)
+  if (tiles > 0 && prompt_kind == 0) {
+    if (kv_rank <= 64) { if (heads >= 4) LM_SHARED(4, 4); else LM_SHARED(4, 1); }
+    else if (kv_rank <= 128) { if (heads >= 4) LM_SHARED(8, 4); else LM_SHARED(8, 1); }
+    else if (kv_rank <= 256) { if (heads >= 2) LM_SHARED(16, 2); else LM_SHARED(16, 1); }
+    else { if (heads >= 2) LM_SHARED(32, 2); else LM_SHARED(32, 1); }
+    TNX_CHECK_LAUNCH("latent_attention_prompt_shared");
+  } else if (tiles > 0) {
     if (kv_rank <= 64) LM_PROMPT(4, 2);
     else if (kv_rank <= 128) LM_PROMPT(8, 2);
     else if (kv_rank <= 256) LM_PROMPT(16, 1);
     else LM_PROMPT(32, 1);
     TNX_CHECK_LAUNCH("latent_attention_prompt");
   }
+#undef LM_SHARED
   if (decodes > 0) {
     if (kv_rank <= 64) LM_DECODE(4);
     else if (kv_rank <= 128) LM_DECODE(8);

@@ -103,7 +103,7 @@ _SIGNATURES = {
         "tnx_latent_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                       _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_void_p,
                                       _c_void_p, _c_void_p, _c_ll, _c_ll, _c_ll, _c_void_p, _c_int, _c_float, _c_int,
-                                      _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
+                                      _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_batched_linear": [_c_void_p, _c_int, _c_ll, _c_ll, _c_void_p, _c_int, _c_void_p, _c_int, _c_float, _c_int,
                                _c_int, _c_int, _c_int, _c_void_p],
         "tnx_latent_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
@@ -1209,6 +1209,7 @@ class HipOps:
         return out
 
     latent_matrix_unit = True      # tests clear it to run the any-sizes kernel in bfloat16 too
+    latent_prompt_kind = 0         # tests set 1: the prompt kernel whose waves each walk the keys for their own queries
 
     def latent_attention(self, q, q_lat, num_heads, head_size, rot, kv_rank, freqs, scale, ctx, view, latent_pages,
                          rotated_pages, across_pages=None, window=None):
@@ -1252,7 +1253,7 @@ class HipOps:
                        _ptr(ctx.plan["decode_runs"]), decodes, _ptr(latent_pages), _ptr(rotated_pages),
                        _ptr(across_pages), latent_pages.stride(0), rotated_pages.stride(0), across_pages.stride(0),
                        _ptr(freqs), freqs.numel(), float(scale), num_heads, head_size, rot, kv_rank, int(window or 0),
-                       _ptr(part), splits, per_split, _stream(),
+                       _ptr(part), splits, per_split, int(self.latent_prompt_kind), _stream(),
                        work=(f"{tiles} tiles {decodes} decodes", seen * (2 * kv_rank + rot) * 2,
                              2.0 * num_heads * (2 * kv_rank + rot) * float(
                                  (ctx.run_lens_host * np.minimum(ctx.cached_lens_host + (ctx.run_lens_host + 1) / 2,
