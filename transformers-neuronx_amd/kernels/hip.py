@@ -529,7 +529,9 @@ class HipOps:
                 taken += size
         return taken
 
-    def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False, force_tiled=False):
+    def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False, force_tiled=False, f32_by_library=False):
+        """`f32_by_library`: a float32 result without a residual may come from the vendor library too (many rows);
+        left False such a product (the head's) stays on our kernel."""
         if isinstance(x, DeferredNorm):
             folded = self._folded_for(x, w) if (residual is None and not out_f32 and force_tiled != 1) else None
             if folded is not None and self._library_product(x.shape[0], w.tensor.shape[0], w.tensor.shape[1],
@@ -613,6 +615,10 @@ class HipOps:
                            _code(out_dtype), m, n, _stream())
             return out
         out = torch.empty(m, n, dtype=out_dtype, device=x.device)
+        if (f32_by_library and out_f32 and residual is None and act in (None, "none") and self.library_direct
+                and self._library_product(m, n, k, w, force_tiled)
+                and self._library_call(self.cast(x, torch.bfloat16), w, bias, None, out, act, m, n, k)):
+            return out
         if w.dtype == torch.float32:
             xa = self.cast(x, torch.float32)
             self._call("gemm", "tnx_gemm_f32", _ptr(xa), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out),
@@ -1048,6 +1054,8 @@ class HipOps:
             return out
         return out, (copy if copy is not None else self.cast(out, self.dtype))
 
+    fuse_rows = 64       # up to this many rows the join, the norm and the convolution are one launch
+
     @staticmethod
     def rows_fit(width: int) -> bool:
         """Whether the kernels that hold a row in registers take this width."""
@@ -1061,7 +1069,9 @@ class HipOps:
         t, width = x.shape
         taps = conv_w.shape[1]
         pw, pb, pc, eps = pre
-        if not self.rows_fit(width):
+        # Many rows: a token's block makes the rows of the taps - 1 tokens before it again, which costs more than
+        # the launches it saves (2,048 rows of 4,096, four taps: 149 us in one launch, 81 in three).
+        if not self.rows_fit(width) or t > self.fuse_rows:
             if join is not None:
                 x = self.norm_add(join[0], join[1], join[2], eps, join[3], x, join[4])
             h = self.layernorm(x, pw, pb, eps, torch.float32, True, False, pc)[0]

@@ -99,7 +99,7 @@ class ReferenceOps:
             return 0.5 * y * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (y + 0.044715 * y * y * y)))
         raise ValueError(f"unknown activation {act!r}")
 
-    def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False):
+    def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False, f32_by_library=False):
         """`act(x w^T + bias) + residual`, `w` being `[out, in]`. An operand in the
         narrower dtype decides what the other is rounded to, except that a
         float32 matrix keeps the product in float32."""

@@ -185,7 +185,7 @@ class SandwichBlock(Block):
                                                                        ctx.kept_tokens)
             g = ops.linear(compute, self.side_gate, None, act="gelu_new")
             g = ops.mul_columns(g, rows, s["offset"])
-            y = ops.linear(g, self.side_proj, None, out_f32=True)
+            y = ops.linear(g, self.side_proj, None, out_f32=True, f32_by_library=True)
             x = ops.norm_add(y, self.side_norm, None, s["eps"], False, x, self.mult, place)
         if not self.depth_average:
             return Stream(x, None)

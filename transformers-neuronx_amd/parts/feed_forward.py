@@ -50,10 +50,11 @@ class DenseFeedForward(FeedForward):
     def forward(self, h, ctx, residual):
         """`residual` None: f(h) alone, in float32 (for an arrangement that norms it before the sum)."""
         if self.activation == "poly_norm":
-            inner = self.ops.poly_norm(self.ops.linear(h, self.w1, self.b1, out_f32=True), self.coeffs, self.eps)
+            inner = self.ops.poly_norm(self.ops.linear(h, self.w1, self.b1, out_f32=True, f32_by_library=True),
+                                       self.coeffs, self.eps)
         else:
             inner = self.ops.linear(h, self.w1, self.b1, act=self.activation)
-        return self.ops.linear(inner, self.w2, self.b2, residual=residual, out_f32=True)
+        return self.ops.linear(inner, self.w2, self.b2, residual=residual, out_f32=True, f32_by_library=residual is None)
 
 
 @register_feed_forward("none")

@@ -227,7 +227,7 @@ class LatentAttention(Mixer):
         if latent.shape[-1] != self.kv_rank or rotated.shape[-1] != r:
             raise ValueError(f"the cache holds latents of {latent.shape[-1]} + {rotated.shape[-1]} elements, "
                              f"this mixer reads {self.kv_rank} + {r}")
-        down = ops.linear(h, self.w_down, None, out_f32=True)
+        down = ops.linear(h, self.w_down, None, out_f32=True, f32_by_library=True)
         c_q = ops.latent_norms(down, self.q_rank, self.kv_rank if self.own_kv else 0, r if self.own_kv else 0,
                                self.q_norm, self.kv_norm, self.eps, self.freqs, ctx, view, latent, rotated, across)
         q = ops.linear(c_q, self.w_uq, None)
@@ -235,4 +235,5 @@ class LatentAttention(Mixer):
         o_lat = ops.latent_attention(q, q_lat, heads, n, r, self.kv_rank, self.freqs, self.scale, ctx, view,
                                      latent, rotated, across, self.window)
         values = ops.batched_linear(o_lat, self.w_uv)
-        return ops.linear(values.view(-1, heads * self.value_size), self.w_o, None, residual=residual, out_f32=True)
+        return ops.linear(values.view(-1, heads * self.value_size), self.w_o, None, residual=residual, out_f32=True,
+                          f32_by_library=residual is None)
