@@ -1,4 +1,4 @@
-"""An inference engine for OPT-family decoders on one AMD MI355X."""
+"""An inference engine for decoder-only language models (OPT, Ratesun) on one AMD MI355X."""
 __version__ = "0.1.0"
 
 from .config import ContinuousBatchingConfig, EngineConfig, GenerationConfig, NeuronConfig  # noqa: F401
@@ -10,6 +10,9 @@ def __getattr__(name):
     if name in ("OPTForSampling", "OPTForGreedySearch"):
         from .opt import model
         return getattr(model, name)
+    if name == "RatesunForSampling":
+        from .ratesun import model
+        return model.RatesunForSampling
     if name == "NeuronAutoModelForCausalLM":
         from .modeling_auto import NeuronAutoModelForCausalLM
         return NeuronAutoModelForCausalLM

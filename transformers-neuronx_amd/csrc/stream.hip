@@ -148,6 +148,40 @@ __device__ __forceinline__ void row_norm(rf4 (&v)[PER], int w4, int width, const
   }
 }
 
+// a vector's chunks as `row_load` lays a row out; zeros for a vector that is not there
+template <int PER>
+__device__ __forceinline__ void vector_load(const float* vec, int w4, float fill, rf4 (&v)[PER]) {
+#pragma unroll
+  for (int c = 0; c < PER; ++c) {
+    const int i = threadIdx.x + 256 * c;
+    v[c] = (vec && i < w4) ? ((const rf4*)vec)[i] : (rf4){fill, fill, fill, fill};
+  }
+}
+
+// `row_norm` with the weight and the bias in registers already (ones and zeros where there is none)
+template <int PER>
+__device__ __forceinline__ void row_norm_held(rf4 (&v)[PER], int w4, int width, const rf4 (&weight)[PER],
+                                              const rf4 (&bias)[PER], float eps, int center, float* scratch) {
+  float s = 0.f;
+  if (center) {
+#pragma unroll
+    for (int c = 0; c < PER; ++c) s += (v[c].x + v[c].y) + (v[c].z + v[c].w);
+  }
+  const float mean = center ? block_sum<4>(s, scratch) / (float)width : 0.f;
+  float q = 0.f;
+#pragma unroll
+  for (int c = 0; c < PER; ++c) {
+    if (threadIdx.x + 256 * c < w4) {
+      const rf4 d = v[c] - mean;
+      q += (d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w);
+    }
+  }
+  const float rstd = 1.f / sqrtf(block_sum<4>(q, scratch) / (float)width + eps);
+#pragma unroll
+  for (int c = 0; c < PER; ++c)
+    if (threadIdx.x + 256 * c < w4) v[c] = (v[c] - mean) * rstd * weight[c] + bias[c];   // (chunks beyond the row stay zero)
+}
+
 __device__ __forceinline__ void store_chunk(void* out, int dtype, size_t chunk, rf4 y) {
   if (dtype == TNX_F32) {
     ((rf4*)out)[chunk] = y;
@@ -187,16 +221,20 @@ norm_add_rows_kernel(const float* __restrict__ y, const float* __restrict__ weig
 // step's run, and come from the request's state otherwise (`[taps, width]`, position p at place p mod taps).
 // `h_keep`: where a run's last taps - 1 tokens leave their h for the launch that writes the state afterwards;
 // with `write_state` (every run of the step is one token) this kernel writes the state itself.
-template <int PER>
+// TAPS: the number of taps where it is 1 to 4 (what is read from the state and the weights are then asked for
+// before the first reduction, and nothing waits for them afterwards); 0: any number, taken as it comes.
+template <int PER, int TAPS>
 __global__ void __launch_bounds__(256)
 join_norm_conv_kernel(const float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ post_w,
                       const float* __restrict__ post_b, int post_center, float mult, float* __restrict__ x_out,
                       const float* __restrict__ pre_w, const float* __restrict__ pre_b, int pre_center, float eps,
-                      const float* __restrict__ conv_w, float* state, size_t slot_stride, int taps,
+                      const float* __restrict__ conv_w, float* state, size_t slot_stride, int taps_given,
                       const int* __restrict__ positions, const int* __restrict__ token_request,
                       const int* __restrict__ run_start, const int* __restrict__ slots, void* __restrict__ out,
                       int out_dtype, float* __restrict__ h_keep, int write_state, int width) {
   __shared__ float scratch[4];
+  const int taps = TAPS > 0 ? TAPS : taps_given;
+  constexpr int KEPT = TAPS > 1 ? TAPS - 1 : 1;
   const int w4 = width >> 2;
   const int t = blockIdx.x;
   const int r = token_request[t];
@@ -206,6 +244,36 @@ join_norm_conv_kernel(const float* __restrict__ x, const float* __restrict__ y, 
   rf4 acc[PER], v[PER];
 #pragma unroll
   for (int c = 0; c < PER; ++c) acc[c] = (rf4){0.f, 0.f, 0.f, 0.f};
+  // the norms' vectors, the taps' weights and what comes from the state, all asked for at once
+  rf4 pw[PER], pb[PER], qw[PER], qb[PER];
+  vector_load<PER>(pre_w, w4, 1.f, pw);
+  vector_load<PER>(pre_b, w4, 0.f, pb);
+  vector_load<PER>(y ? post_w : nullptr, w4, 1.f, qw);
+  vector_load<PER>(y ? post_b : nullptr, w4, 0.f, qb);
+  rf4 taps_w[TAPS > 0 ? TAPS : 1][PER];
+  if (TAPS > 0) {
+#pragma unroll
+    for (int j = 0; j < (TAPS > 0 ? TAPS : 1); ++j)
+#pragma unroll
+      for (int c = 0; c < PER; ++c) {
+        const int k = threadIdx.x + 256 * c;
+        const float* cw = conv_w + (size_t)(4 * min(k, w4 - 1)) * TAPS + j;
+        taps_w[j][c] = (rf4){cw[0], cw[TAPS], cw[2 * TAPS], cw[3 * TAPS]};
+      }
+  }
+  rf4 kept[KEPT][PER];
+  if (TAPS > 1) {
+#pragma unroll
+    for (int back = 1; back < (TAPS > 1 ? TAPS : 1); ++back) {
+      if (back > i && back <= p && mine) {
+        row_load<PER>(mine + (size_t)((p - back) % taps) * width, w4, kept[back - 1]);
+      } else {
+#pragma unroll
+        for (int c = 0; c < PER; ++c) kept[back - 1][c] = (rf4){0.f, 0.f, 0.f, 0.f};
+      }
+    }
+  }
+#pragma unroll 1
   for (int back = taps - 1; back >= 0; --back) {
     if (back <= i) {
       const size_t row = (size_t)(t - back) * width;
@@ -213,7 +281,7 @@ join_norm_conv_kernel(const float* __restrict__ x, const float* __restrict__ y, 
       if (y) {
         rf4 u[PER];
         row_load<PER>(y + row, w4, u);
-        row_norm<PER>(u, w4, width, post_w, post_b, eps, post_center, scratch);
+        row_norm_held<PER>(u, w4, width, qw, qb, eps, post_center, scratch);
 #pragma unroll
         for (int c = 0; c < PER; ++c) {
           v[c] = v[c] + mult * u[c];
@@ -221,7 +289,15 @@ join_norm_conv_kernel(const float* __restrict__ x, const float* __restrict__ y, 
           if (back == 0 && k < w4) ((rf4*)(x_out + row))[k] = v[c];
         }
       }
-      row_norm<PER>(v, w4, width, pre_w, pre_b, eps, pre_center, scratch);
+      row_norm_held<PER>(v, w4, width, pw, pb, eps, pre_center, scratch);
+    } else if (TAPS > 1) {
+      if (back > p) continue;
+#pragma unroll
+      for (int b = 1; b < (TAPS > 1 ? TAPS : 1); ++b)
+        if (b == back) {
+#pragma unroll
+          for (int c = 0; c < PER; ++c) v[c] = kept[b - 1][c];
+        }
     } else if (back <= p && mine) {
       row_load<PER>(mine + (size_t)((p - back) % taps) * width, w4, v);
     } else {
@@ -232,8 +308,16 @@ join_norm_conv_kernel(const float* __restrict__ x, const float* __restrict__ y, 
     for (int c = 0; c < PER; ++c) {
       const int k = threadIdx.x + 256 * c;
       if (k < w4) {
-        const float* cw = conv_w + (size_t)(4 * k) * taps + j;
-        const rf4 wj = {cw[0], cw[taps], cw[2 * taps], cw[3 * taps]};
+        rf4 wj;
+        if (TAPS > 0) {
+          wj = taps_w[0][c];
+#pragma unroll
+          for (int jj = 1; jj < (TAPS > 0 ? TAPS : 1); ++jj)
+            if (jj == j) wj = taps_w[jj][c];
+        } else {
+          const float* cw = conv_w + (size_t)(4 * k) * taps + j;
+          wj = (rf4){cw[0], cw[taps], cw[2 * taps], cw[3 * taps]};
+        }
         acc[c] = acc[c] + wj * v[c];
         if (back == 0) acc[c] = acc[c] + v[c];
       }
@@ -327,13 +411,19 @@ extern "C" int tnx_join_norm_conv(const float* x, const float* y, const float* p
   TNX_REQUIRE(taps == 1 || single_runs || h_keep, "join_norm_conv: nowhere to leave the inputs that the state takes");
   TNX_REQUIRE(!y || (x_out && x_out != x), "join_norm_conv: the joined stream needs a place of its own");
   if (tokens == 0) return 0;
-#define JN_LAUNCH(PER)                                                                                                \
-  join_norm_conv_kernel<PER><<<tokens, 256, 0, stream>>>(x, y, post_w, post_b, post_center, mult, x_out, pre_w, pre_b, \
-                                                         pre_center, eps, conv_w, taps > 1 ? state : nullptr,          \
-                                                         (size_t)slot_stride, taps, positions, token_request,          \
-                                                         run_start, slots, out, out_dtype, h_keep, single_runs, width)
+#define JN_ARGS                                                                                                       \
+  x, y, post_w, post_b, post_center, mult, x_out, pre_w, pre_b, pre_center, eps, conv_w, taps > 1 ? state : nullptr,  \
+      (size_t)slot_stride, taps, positions, token_request, run_start, slots, out, out_dtype, h_keep, single_runs, width
+#define JN_LAUNCH(PER)                                                                       \
+  switch (taps) {                                                                            \
+    case 2: join_norm_conv_kernel<PER, 2><<<tokens, 256, 0, stream>>>(JN_ARGS); break;       \
+    case 3: join_norm_conv_kernel<PER, 3><<<tokens, 256, 0, stream>>>(JN_ARGS); break;       \
+    case 4: join_norm_conv_kernel<PER, 4><<<tokens, 256, 0, stream>>>(JN_ARGS); break;       \
+    default: join_norm_conv_kernel<PER, 0><<<tokens, 256, 0, stream>>>(JN_ARGS); break;      \
+  }
   ROWS_DISPATCH(width, JN_LAUNCH)
 #undef JN_LAUNCH
+#undef JN_ARGS
   TNX_CHECK_LAUNCH("join_norm_conv");
   if (taps > 1 && !single_runs) {
     conv_state_kernel<<<dim3((width + 255) / 256, runs), 256, 0, stream>>>(h_keep, state, (size_t)slot_stride, taps,
