@@ -400,3 +400,21 @@ def test_the_replay_program_serves_a_folder(tmp_path):
         got = np.fromfile(out_dir / f"{step}.f32", dtype="<f4").reshape(-1, cfg.vocab)[row]
         want = expected[rid][pos].numpy()
         assert np.abs(got - want).max() / np.abs(expected[rid].numpy()).max() < 2e-5
+
+
+def test_the_command_line_serves_the_folder(tmp_path, capsys):
+    """`opt_demo save --random --config` writes a folder of whatever architecture the config.json names, and
+    `run --benchmark --profile` generates from it and times its kernels."""
+    from transformers_neuronx_amd.opt import demo
+    with open(tmp_path / "config.json", "w") as fp:
+        json.dump(dict(rc.CASES["d"], init_std=0.3), fp)
+    folder = str(tmp_path / "model")
+    assert demo.main(["--amp", "bf16", "save", folder, "--random", "--config", str(tmp_path / "config.json")]) in (0, None)
+    assert demo.main(["--amp", "bf16", "run", folder, "--batch_size", "2", "--n_positions", "40", "--prompt_len", "9",
+                      "--top_k", "1", "--benchmark", "--profile", "--page_size", "16"]) in (0, None)
+    text = capsys.readouterr().out
+    assert "running RatesunForSampling.from_pretrained" in text
+    report = json.loads(next(line for line in text.splitlines() if line.startswith("{")))
+    assert report["inferences"] == 10 and report["e2e_output_token_throughput"] > 0
+    for kernel in ("tnx_join_norm_conv", "tnx_latent_attention_mfma", "tnx_batched_linear", "tnx_poly_norm", "tnx_embed_pairs"):
+        assert kernel in text, kernel

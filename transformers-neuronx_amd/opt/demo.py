@@ -93,7 +93,7 @@ def save(args):
 
 def run(args):
     from ..config.engine_config import GenerationConfig
-    from .model import OPTForSampling
+    from ..modeling_auto import NeuronAutoModelForCausalLM
     if args.quantize:
         raise SystemExit("run: --quantize is not to be had here: weights stay in the dtype of --amp")
     torch.manual_seed(args.seed)
@@ -101,14 +101,16 @@ def run(args):
         # generation_demo.py:551-554 names the folder in the environment, where the runtime looks for it
         os.environ["TNX_SNAPSHOT_PATH"] = f"tnx_snapshot_{args.amp}_b{args.batch_size}"
         print(f"Set snapshot path {os.environ['TNX_SNAPSHOT_PATH']}")
-    print("running OPTForSampling.from_pretrained")
-    model = OPTForSampling.from_pretrained(args.load, batch_size=args.batch_size, amp=args.amp,
-                                           tp_degree=args.tp_degree, n_positions=args.n_positions,
-                                           unroll=args.unroll, context_length_estimate=args.context_length_estimate,
-                                           page_size=args.page_size)
+    # the class is the one the folder's config.json names (OPT's, or that of any registered architecture)
+    model = NeuronAutoModelForCausalLM.from_pretrained(args.load, batch_size=args.batch_size, amp=args.amp,
+                                                       tp_degree=args.tp_degree, n_positions=args.n_positions,
+                                                       unroll=args.unroll,
+                                                       context_length_estimate=args.context_length_estimate,
+                                                       page_size=args.page_size)
+    print(f"running {type(model).__name__}.from_pretrained")
     print("running model.load")
     model.load()
-    vocab = model.config.vocab_size
+    vocab = model.architecture.build_spec(model.config).vocab_size
     if args.prompt_ids:
         row = [int(t) for t in args.prompt_ids.split(",")]
         input_ids = torch.tensor([row] * args.batch_size)

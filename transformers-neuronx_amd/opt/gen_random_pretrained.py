@@ -1,4 +1,4 @@
-"""Write an OPT model folder with random weights.
+"""Write a model folder with random weights: OPT's, or that of any registered architecture whose config.json is given.
 
     opt_gen_random_pretrained NAME SAVE [--seed N] [--dtype DTYPE]
 
@@ -33,7 +33,10 @@ def gen_random_pretrained(model_name: str, save: str, seed: int = 0, dtype=None)
             raise FileNotFoundError(f"{model_name}: no such config.json (there is no network to fetch a model name)")
         with open(path) as fp:
             raw = json.load(fp)
-    return write_random_model(OPTConfig.from_dict(raw), save, seed, dtype)
+    from ..config.registry import resolve
+    names_one = raw.get("architectures") or raw.get("architecture") or raw.get("model_type")
+    config_class = resolve(raw).config_class if names_one else OPTConfig      # a bare OPT config.json names none
+    return write_random_model(config_class.from_dict(raw), save, seed, dtype)
 
 
 def main(argv=None):
