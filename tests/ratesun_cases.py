@@ -83,3 +83,38 @@ def runner(cfg, w, dtype="float32", kernels="reference", device="cpu", page_size
 def requests(cfg, lengths, seed):
     g = torch.Generator().manual_seed(seed)
     return {f"r{i}": torch.randint(0, cfg.vocab, (n,), generator=g).tolist() for i, n in enumerate(lengths)}
+
+
+def drawn(seed: int) -> RatesunConfig:
+    """A configuration drawn from a seed: any sizes, any order of layers with and without a latent of their own,
+    with and without a feed-forward, windows from 1 token to none."""
+    import random
+    rnd = random.Random(seed)
+    width = rnd.choice([24, 36, 64, 100, 128, 256])
+    n_layers = rnd.randint(1, 5)
+    layers, own = [], []
+    for i in range(n_layers):
+        window = rnd.choice([None, 1, 2, 7, 16, 17, 31, 48, 64, 65, 90])
+        base = rnd.choice([10.0, 500.0, 10000.0, 1e6])
+        if own and rnd.random() < 0.45:
+            src = rnd.choice(own)
+            of = layers[src]["mixer"]
+            m = _mixer(rnd.randint(1, 6), rnd.choice([4, 8, 10, 16, 32]), of["rot_dim"], rnd.choice([4, 6, 16, 24]),
+                       of["kv_rank"], rnd.choice([8, 12, 32, 40]), window, of["rot"]["base"], rnd.uniform(0.05, 0.4),
+                       kv_from=src, dims=of["rot"]["dims"])
+        else:
+            rot = rnd.choice([2, 4, 8, 16])
+            m = _mixer(rnd.randint(1, 6), rnd.choice([4, 8, 10, 16, 32]), rot, rnd.choice([4, 6, 16, 24]),
+                       rnd.choice([8, 16, 20, 32, 48, 64]), rnd.choice([8, 12, 32, 40]), window, base,
+                       rnd.uniform(0.05, 0.4), dims=rnd.choice([rot, max(2, rot - 2)]))
+            own.append(i)
+        layers.append(_layer(m, rnd.choice([None, 16, 40, 72, 130]) if n_layers > 1 else 40))
+    raw = dict(architecture="Ratesun", vocab=rnd.choice([50, 97, 256, 300]), width=width, norm=dict(eps=rnd.choice([1e-6, 1e-5, 1e-3])),
+               residual_mult=rnd.uniform(0.2, 1.0), logit_scale=rnd.uniform(0.25, 2.0), layers=layers, init_std=0.35)
+    if rnd.random() < 0.8:
+        raw["canon"] = dict(taps=rnd.randint(1, 5))
+    if rnd.random() < 0.8:
+        raw["embedding"] = dict(bigram=dict(buckets=rnd.choice([1, 7, 64, 1021]), mul_prev=rnd.randint(0, 2000), mul_cur=rnd.randint(1, 50)))
+    if rnd.random() < 0.8:
+        raw["token_side"] = dict(dim=rnd.choice([1, 4, 5, 16]))
+    return RatesunConfig.from_dict(raw)

@@ -85,7 +85,10 @@ def test_config_reads_the_nested_keys_and_names_the_one_at_fault(tmp_path):
     assert [(c.layer, c.cache, c.writes) for c in spec.schedule] == [(0, 0, True), (1, 0, False), (2, 2, True), (3, 2, False)]
     # the latent of layer 0 is kept for the wider window of its reader, that of layer 2 for good
     assert spec.layers[0].mixer.params["keep"] == 50 and spec.layers[0].mixer.params["window"] == 24
-    assert spec.layers[2].mixer.params["keep"] is None
+    assert spec.layers[2].mixer.params["keep"] == "all"
+    # a writer with a window whose reader sees everything keeps everything (seed 1 of the drawn configurations)
+    drawn = ratesun_spec(rc.drawn(1))
+    assert drawn.layers[0].mixer.params["window"] == 1 and drawn.layers[0].mixer.params["keep"] == "all"
     folder = write_random_model(cfg, str(tmp_path / "m"), 0, dtype="float32")
     arch, read = read_config(folder)
     assert arch.name == "Ratesun" and read.layers == cfg.layers and read.to_dict() == dict(cfg.to_dict(), torch_dtype="float32")
@@ -135,18 +138,26 @@ def _expected(cfg, w, requests):
     return {rid: P.forward(raw, wide, toks) for rid, toks in requests.items()}
 
 
-def step_through(runner, expected, made, tol):
+def step_through(runner, expected, made, tol, few_over=0.0):
+    """`few_over`: the share of positions that may lie over `tol` (none by more than ten times): bfloat16 at a
+    place where the model itself is ill-conditioned, such as a token-keyed input of one element, whose sign a
+    rounding can turn; the plain implementation in bfloat16 arithmetic is as far off there."""
     steps, place = made
+    over, seen = [], 0
     for rec in steps:
         logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in rec["entries"]])
         for row in range(0 if logits is None else logits.shape[0]):
             rid, pos = place[(rec["step"], row)]
             want = expected[rid][pos]
             err = float((logits[row].double().cpu() - want).abs().max() / expected[rid].abs().max())
-            assert err < tol, (rec["step"], rid, pos, err)
+            seen += 1
+            if not err < tol:
+                over.append((rec["step"], rid, pos, err))
+            assert err < tol * (10 if few_over else 1), (rec["step"], rid, pos, err)
         for rid in rec["end"]:
             runner.finish(rid)
         runner.cache.check()
+    assert len(over) <= few_over * seen, over[:5]
     assert not runner.cache.requests
 
 
@@ -248,3 +259,12 @@ def test_bindings_pass_as_many_arguments_as_the_entry_points_take():
             found = re.search(r'extern "C" int ' + name + r"\(([^)]*)\)", source)
             assert found, f"{module}.hip has no entry point {name}"
             assert len([a for a in found.group(1).split(",") if a.strip()]) == len(types), name
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_configurations_drawn_from_a_seed_on_the_host(seed):
+    cfg = rc.drawn(seed)
+    w = rc.weights(cfg, seed)
+    runner = rc.runner(cfg, w, max_tokens=176)
+    requests = rc.requests(cfg, [70, 33, 5, 1], seed)
+    step_through(runner, _expected(cfg, w, requests), schedules.mixed(requests, max_tokens=176, page=16, seed=5, tail=8, max_live=3), 2e-5)

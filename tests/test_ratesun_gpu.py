@@ -418,3 +418,16 @@ def test_the_command_line_serves_the_folder(tmp_path, capsys):
     assert report["inferences"] == 10 and report["e2e_output_token_throughput"] > 0
     for kernel in ("tnx_join_norm_conv", "tnx_latent_attention_mfma", "tnx_batched_linear", "tnx_poly_norm", "tnx_embed_pairs"):
         assert kernel in text, kernel
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 6e-2)])
+@pytest.mark.parametrize("seed", range(12))
+def test_configurations_drawn_from_a_seed(seed, dtype, tol):
+    cfg = rc.drawn(seed)
+    w = rc.weights(cfg, seed, torch.bfloat16 if dtype == "bfloat16" else torch.float32)
+    runner = rc.runner(cfg, w, dtype=dtype, kernels="hip", device=DEV, max_tokens=176)
+    requests = rc.requests(cfg, [70, 33, 5, 1], seed)
+    expected = _expected(cfg, w, requests)
+    few = 0.03 if dtype == "bfloat16" else 0.0
+    step_through(runner, expected, schedules.mixed(requests, max_tokens=176, page=16, seed=5, tail=8, max_live=3), tol, few)
+    step_through(runner, expected, schedules.head_then_singles(requests, tail=20), tol, few)

@@ -143,22 +143,24 @@ class LatentAttention(Mixer):
     values are: the weighted sum contracts over tokens, and the matrix unit wants them next to each other.
 
     `own_kv=False`: no W_dkv; the mixer reads the cache of another call of the run order, whose R, r and
-    rotation are its own. `keep`: the tokens the cache keeps (None: all); a cache that is read by mixers of
-    different windows keeps the most any of them sees.
+    rotation are its own. `keep`: the tokens the cache keeps: a number, "all", or None for the mixer's own window;
+    a cache that is read by mixers of different windows keeps the most any of them sees.
     """
 
     recordable = True
 
     def __init__(self, width: int, num_heads: int, head_size: int, rot_size: int, value_size: int, kv_rank: int,
                  q_rank: int, scale: float, eps: float, rotation, names, window: Optional[int] = None,
-                 keep: Optional[int] = None, own_kv: bool = True, norm_suffix: str = ".norm", weight_suffix: str = ""):
+                 keep=None, own_kv: bool = True, norm_suffix: str = ".norm", weight_suffix: str = ""):
         """`names`: the checkpoint's names, relative to the mixer's prefix, of W_dq, W_uq, W_dkv, W_uk, W_uv and
         W_o; a latent's norm weight is its down-projection's name with `norm_suffix`."""
         self.width, self.num_heads, self.head_size, self.rot_size = width, num_heads, head_size, rot_size
         self.value_size, self.kv_rank, self.q_rank = value_size, kv_rank, q_rank
         self.scale, self.eps, self.window, self.own_kv = float(scale), float(eps), window, own_kv
         self.keep = keep if own_kv else None
-        if own_kv and window is not None and keep is not None and keep < window:
+        if keep is not None and keep != "all" and (not isinstance(keep, int) or keep < 1):
+            raise ValueError(f"keep is a number of tokens, \"all\" or None, got {keep!r}")
+        if own_kv and isinstance(keep, int) and (window is None or keep < window):
             raise ValueError(f"a cache that keeps {keep} tokens cannot serve a window of {window}")
         self.names = tuple(names)
         if len(self.names) != 6:
@@ -169,7 +171,7 @@ class LatentAttention(Mixer):
             raise ValueError(f"the rotated part has {rot_size} elements; the rotation turns {self.rotation.dims}")
 
     def cache_need(self) -> Optional[CacheNeed]:
-        keep = self.keep if self.keep is not None else self.window
+        keep = None if self.keep == "all" else (self.keep if self.keep is not None else self.window)
         return CacheNeed("paged", window=keep,
                          page_tensors=(("latent", ("page", self.kv_rank)), ("rotated", ("page", self.rot_size)),
                                        ("across", (self.kv_rank, "page"))))

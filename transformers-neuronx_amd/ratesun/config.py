@@ -99,10 +99,11 @@ class RatesunConfig(ModelConfig):
             m = layer.get("mixer")
             for key in ("heads", "dim", "rot_dim", "vdim", "kv_rank", "q_rank"):
                 _need(m, key, int, where + ".mixer")
-            _need(m, "scale", float, where + ".mixer")
+            if "scale" in m:
+                _need(m, "scale", float, where + ".mixer")
             rot = m.get("rot")
             _need(rot, "base", float, where + ".mixer.rot")
-            dims = _need(rot, "dims", int, where + ".mixer.rot")
+            dims = _need(rot, "dims", int, where + ".mixer.rot") if "dims" in rot else m["rot_dim"]
             if dims % 2 or dims > m["rot_dim"]:
                 raise ConfigError(f"key '{where}.mixer.rot.dims' ({dims}) must be even and at most rot_dim ({m['rot_dim']})")
             if m.get("mask") is not None:

@@ -20,20 +20,24 @@ def ratesun_spec(cfg: RatesunConfig) -> ModelSpec:
     keeps = {}
     for i, layer in enumerate(cfg.layers):
         m = layer["mixer"]
-        src = m.get("kv_from", i) if m.get("kv_from") is not None else i
-        size = (m.get("mask") or {}).get("size")
+        src = m["kv_from"] if m.get("kv_from") is not None else i
+        size = (m.get("mask") or {}).get("size") or "all"
         if src not in keeps:
             keeps[src] = size
-        elif keeps[src] is not None:
-            keeps[src] = None if size is None else max(keeps[src], size)
+        elif keeps[src] != "all":
+            keeps[src] = "all" if size == "all" else max(keeps[src], size)
     layers, schedule, unread = [], [], []
     for i, layer in enumerate(cfg.layers):
         m = layer["mixer"]
         own = m.get("kv_from") is None
         mixer = PartSpec("latent_attention", dict(
             width=d, num_heads=m["heads"], head_size=m["dim"], rot_size=m["rot_dim"], value_size=m["vdim"],
-            kv_rank=m["kv_rank"], q_rank=m["q_rank"], scale=m["scale"], eps=cfg.eps,
-            rotation=PartSpec("rotary", dict(base=m["rot"]["base"], dims=m["rot"]["dims"], interleaved=True)),
+            kv_rank=m["kv_rank"], q_rank=m["q_rank"], eps=cfg.eps,
+            # a mixer that names no scale gets the usual one for its query/key size; one that names no number of
+            # turned elements turns the whole rotated part
+            scale=m.get("scale", (m["dim"] + m["rot_dim"]) ** -0.5),
+            rotation=PartSpec("rotary", dict(base=m["rot"]["base"], dims=m["rot"].get("dims", m["rot_dim"]),
+                                             interleaved=True)),
             names=MIX_NAMES, window=(m.get("mask") or {}).get("size"), keep=keeps[i] if own else None, own_kv=own))
         mlp = layer.get("mlp")
         if mlp is not None:
