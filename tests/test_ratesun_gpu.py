@@ -431,3 +431,72 @@ def test_configurations_drawn_from_a_seed(seed, dtype, tol):
     few = 0.03 if dtype == "bfloat16" else 0.0
     step_through(runner, expected, schedules.mixed(requests, max_tokens=176, page=16, seed=5, tail=8, max_live=3), tol, few)
     step_through(runner, expected, schedules.head_then_singles(requests, tail=20), tol, few)
+
+
+@pytest.mark.parametrize("case", [
+    dict(heads=3, n=16, r=8, v=32, R=48, window=40, length=300, run=150, ps=16, back=39),
+    dict(heads=3, n=16, r=8, v=32, R=48, window=40, length=300, run=150, ps=16, back=40),
+    dict(heads=2, n=64, r=32, v=64, R=128, window=0, length=700, run=300, ps=64, back=699),
+    dict(heads=5, n=8, r=8, v=16, R=24, window=17, length=64, run=64, ps=16, back=16),
+    dict(heads=1, n=128, r=64, v=128, R=512, window=100, length=400, run=130, ps=64, back=99),
+    dict(heads=2, n=24, r=16, v=48, R=40, window=300, length=280, run=2, ps=16, back=279),
+])
+def test_prompt_attention_with_keys_and_values_made_explicitly(case):
+    """bfloat16 steps of prompts' runs alone: keys W_uk c and values W_uv c of what a run can see are made from
+    the cached latents and attention runs on them. One key is made to stand out for the last query."""
+    from transformers_neuronx_amd.kernels.attention_plan import attention_plan
+    dtype = torch.bfloat16
+    ops = _ops(dtype)
+    heads, n, r, v, R, window, length, run, ps = (case[k] for k in ("heads", "n", "r", "v", "R", "window", "length", "run", "ps"))
+    standout = length - 1 - case["back"]
+    g = torch.Generator().manual_seed(9)
+    w_uk = (torch.randn(heads * n, R, generator=g) / R ** 0.5).to(dtype)
+    w_uv = (torch.randn(heads * v, R, generator=g) / R ** 0.5).to(dtype)
+    c = torch.randn(length, R, generator=g).to(dtype)
+    kr = torch.randn(length, r, generator=g).to(dtype)
+    q = torch.randn(run, heads, n + r, generator=g).to(dtype) * 0.3
+    keys = (c.double() @ w_uk.double().T).view(length, heads, n)
+    q[-1, :, :n] = (keys[standout] / keys[standout].norm(dim=-1, keepdim=True) * 12).to(dtype)
+    c[standout] = c[standout] * 4
+    blocks = -(-length // ps)
+    order = torch.randperm(blocks + 3, generator=g)[:blocks].tolist()
+    lat = torch.randn(blocks + 3, ps, R, generator=g).to(dtype).to(DEV) * 50
+    rot = torch.randn(blocks + 3, ps, r, generator=g).to(dtype).to(DEV) * 50
+    for j in range(length):
+        lat[order[j // ps], j % ps] = c[j]
+        rot[order[j // ps], j % ps] = kr[j]
+    dims, base, scale = r - 2, 321.0, 0.4
+    freqs = (base ** (-2.0 * torch.arange(dims // 2, dtype=torch.float64) / dims)).float().to(DEV)
+    # the mechanism restated with keys and values made explicitly, in float64
+    cd, pos = c.double(), torch.arange(length - run, length)
+    keys = (cd @ w_uk.double().T).view(length, heads, n)
+    vals = (cd @ w_uv.double().T).view(length, heads, v)
+    q_r = P.rotate_pairs(q.double()[..., n:], pos, base, dims)
+    scores = (torch.einsum("ihd,jhd->hij", q.double()[..., :n], keys) + torch.einsum("ihd,jd->hij", q_r, kr.double())) * scale
+    i, j = pos[:, None], torch.arange(length)[None, :]
+    seen = (j <= i) & ((i - j < window) if window else torch.ones_like(j <= i))
+    prob = torch.softmax(scores.masked_fill(~seen[None], float("-inf")), dim=-1)
+    want = torch.einsum("hij,jhd->ihd", prob, vals).reshape(run, heads * v)
+    visible = not window or case["back"] < window
+    assert (float(prob[:, -1, standout].min()) > 0.9) == visible
+    ctx = build_context([StepEntry(0, [0] * run, [])], [length - run], [0], {"g": np.asarray([order], dtype=np.int32)}, ps, DEV,
+                        {"attention": attention_plan})
+    ops.expand_rows = 2
+    assert ops.latent_expands(ctx, n, r, v, R)
+    got = ops.latent_attention_expanded(q.reshape(run, -1).to(DEV), w_uk.to(DEV), w_uv.to(DEV), heads, n, r, v, R, freqs, scale,
+                                        ctx, ctx.groups["g"], lat, rot, window or None)
+    _close(got, want, 2e-2)
+
+
+@pytest.mark.parametrize("name", ["d"])
+def test_schedules_with_expanded_prompt_steps(name):
+    """The engine in bfloat16 with every step of prompts' runs alone on the expanded keys and values."""
+    cfg = rc.config(name)
+    w = rc.weights(cfg, 3, torch.bfloat16)
+    runner = rc.runner(cfg, w, dtype="bfloat16", kernels="hip", device=DEV, max_tokens=400)
+    runner.ops.expand_rows = 2
+    requests = rc.requests(cfg, [170, 33, 5, 100, 2], 1)
+    expected = _expected(cfg, w, requests)
+    for made in (schedules.whole(requests), schedules.portions(requests),
+                 schedules.mixed(requests, max_tokens=400, page=16, seed=5, tail=8, max_live=3)):
+        step_through(runner, expected, made, 6e-2)

@@ -972,3 +972,239 @@ extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void*
 #undef LM_DECODE
   return 0;
 }
+
+// ------------------------------------------------------------------------------------------------ prompts, keys expanded
+
+// For steps that are prompts' runs only, the other order of the products pays: the keys W_uk c and the values
+// W_uv c of the tokens a run can see are made once a step by library products (from the latents gathered out of
+// the pages into dense rows), and attention runs on them as on ordinary keys and values: a (query, key) pair
+// then costs 2 (n + r + v) multiply-adds a head instead of 2 (2 R + r).
+
+// row i of the dense latents: the token at `row_pos[i]` of run `row_run[i]` (zeros for a row that pads a run)
+__global__ void __launch_bounds__(256)
+latent_gather_kernel(const bf16_t* __restrict__ latent_pages, const bf16_t* __restrict__ rotated_pages,
+                     size_t latent_stride, size_t rotated_stride, int page_size, int num_pages,
+                     const int* __restrict__ table, int table_width, const int* __restrict__ row_run,
+                     const int* __restrict__ row_pos, bf16_t* __restrict__ c_dense, bf16_t* __restrict__ r_dense,
+                     int kv_rank, int rot) {
+  const int i = blockIdx.x;
+  const int pos = row_pos[i];
+  int page = -1;
+  if (pos >= 0) {
+    const int b = pos / page_size;
+    page = b < table_width ? table[(size_t)row_run[i] * table_width + b] : -1;
+    if (page >= num_pages) page = -1;
+  }
+  const bf16_t* c = page >= 0 ? latent_pages + (size_t)page * latent_stride + (size_t)(pos % page_size) * kv_rank : nullptr;
+  const bf16_t* kr = page >= 0 ? rotated_pages + (size_t)page * rotated_stride + (size_t)(pos % page_size) * rot : nullptr;
+  for (int d = threadIdx.x; d < kv_rank; d += 256) c_dense[(size_t)i * kv_rank + d] = c ? c[d] : (bf16_t)0.f;
+  for (int d = threadIdx.x; d < rot; d += 256) r_dense[(size_t)i * rot + d] = kr ? kr[d] : (bf16_t)0.f;
+}
+
+// One block: 64 consecutive queries of one head of one run (QB = 4 blocks of 16 columns). Its four waves work on
+// the same 64-key tile: each the scores of 16 keys for all columns, then each a quarter of the value's blocks of
+// 16 elements over all 64 keys. `k_n` `[rows, heads * n]`, `k_r` `[rows, rot]` (turned already), `v_t`
+// `[heads * v, rows]` (a head's values with the tokens side by side); a run's rows begin at `ctx_start[run]`
+// with the token at position `ctx_base[run]` (both multiples of 64).
+template <int NKS, int NDV>
+__global__ void __launch_bounds__(256)
+expanded_attention_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_n, const bf16_t* __restrict__ k_r,
+                          const bf16_t* __restrict__ v_t, bf16_t* __restrict__ out, const int* __restrict__ run_start,
+                          const int* __restrict__ cached_lens, const int* __restrict__ ctx_start,
+                          const int* __restrict__ ctx_base, const int* __restrict__ tile_run,
+                          const int* __restrict__ tile_q0, int tile_tokens, size_t rows, const float* __restrict__ freqs,
+                          int pairs, float scale, int heads, int head_size, int rot, int value_size, int window) {
+  constexpr int QB = 4;
+  constexpr int OWN = (NDV + 3) / 4;
+  __shared__ float tile_max[4][QB][16], tile_sum[4][QB][16];
+  __shared__ __attribute__((aligned(16))) bf16_t prob[QB][16][64 + 8];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int parts = tile_tokens / (16 * QB);
+  const int h = blockIdx.x % heads;
+  const int part = (blockIdx.x / heads) % parts, tile = blockIdx.x / heads / parts;
+  const int run = tile_run[tile];
+  const int t0 = run_start[run], qlen = run_start[run + 1] - t0, cached = cached_lens[run];
+  const int q0 = tile_q0[tile] + 16 * QB * part;
+  if (q0 >= qlen) return;
+  const int total = cached + qlen;
+  const int base = ctx_base[run];
+  const size_t first_row = (size_t)ctx_start[run];
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int qk = head_size + rot;
+
+  bf16x8 qf[QB][NKS];
+  int qpos[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    const int qi = q0 + 16 * qb + r;
+    qpos[qb] = cached + qi;
+    const bf16_t* qrow = q + ((size_t)(t0 + min(qi, qlen - 1)) * heads + h) * qk;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks)
+      qf[qb][ks] = latent_query_chunk(qrow, qrow + head_size, 32 * ks + 8 * g, head_size, rot, qpos[qb], freqs, pairs);
+  }
+  const int first_q = cached + q0, last_q = cached + min(q0 + 16 * QB - 1, qlen - 1);
+  const int lo = max(base, window > 0 ? max(0, first_q - window + 1) : 0);
+  float m[QB], l[QB];
+  f32x4 o[OWN][QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    m[qb] = -INFINITY;
+    l[qb] = 0.f;
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) o[j][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+  for (int tile0 = (lo / 64) * 64; tile0 <= last_q; tile0 += 64) {
+    const int key0 = tile0 + 16 * wave;
+    f32x4 a[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) a[qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const bool live = key0 <= last_q;
+    if (live) {
+      const size_t row = first_row + (size_t)(key0 - base + r);
+      const bf16_t* krow = k_n + (row * heads + h) * head_size;
+      const bf16_t* rrow = k_r + row * rot;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int d0 = 32 * ks + 8 * g;
+        bf16x8 kf = zero8;
+        if (d0 < head_size) kf = *(const bf16x8*)(krow + d0);
+        else if (d0 < qk) kf = *(const bf16x8*)(rrow + (d0 - head_size));
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) a[qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qb][ks], a[qb], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = key0 + 4 * g + i;
+        const bool ok = live && key <= qpos[qb] && (window <= 0 || key > qpos[qb] - window);
+        a[qb][i] = ok ? a[qb][i] * scale : -INFINITY;
+        mx = fmaxf(mx, a[qb][i]);
+      }
+      mx = rows_max(mx);
+      if (g == 0) tile_max[wave][qb][r] = mx;
+    }
+    __syncthreads();
+    float alpha[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      const float m_new = fmaxf(m[qb], fmaxf(fmaxf(tile_max[0][qb][r], tile_max[1][qb][r]),
+                                             fmaxf(tile_max[2][qb][r], tile_max[3][qb][r])));
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      alpha[qb] = __expf(m[qb] - m_safe);
+      m[qb] = m_new;
+      float sum = 0.f;
+      bf16x4 p4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pr = __expf(a[qb][i] - m_safe);
+        sum += pr;
+        p4[i] = (bf16_t)pr;
+      }
+      sum = rows_sum(sum);
+      *(bf16x4*)&prob[qb][r][16 * wave + 4 * g] = p4;
+      if (g == 0) tile_sum[wave][qb][r] = sum;
+    }
+    __syncthreads();
+    bf16x8 pb[QB][2];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      l[qb] = l[qb] * alpha[qb] + ((tile_sum[0][qb][r] + tile_sum[1][qb][r]) + (tile_sum[2][qb][r] + tile_sum[3][qb][r]));
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) pb[qb][s2] = *(const bf16x8*)&prob[qb][r][32 * s2 + 8 * g];
+    }
+    const bool tail = tile0 + 64 > total;
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) {
+      const int db = wave + 4 * j;
+      if (16 * db >= value_size) continue;
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[j][qb][i] *= alpha[qb];
+      const bf16_t* vrow = v_t + ((size_t)h * value_size + 16 * db + r) * rows + first_row + (size_t)(tile0 - base);
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        bf16x8 vf = zero8;
+        if (tile0 + 32 * s2 <= last_q) vf = *(const bf16x8*)(vrow + 32 * s2 + 8 * g);
+        if (tail) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (tile0 + 32 * s2 + 8 * g + e >= total) vf[e] = 0;
+        }
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) o[j][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[qb][s2], o[j][qb], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    const int qi = q0 + 16 * qb + r;
+    if (qi >= qlen) continue;
+    const float inv = l[qb] > 0.f ? 1.f / l[qb] : 0.f;
+    bf16_t* orow = out + ((size_t)(t0 + qi) * heads + h) * value_size;
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) {
+      const int db = wave + 4 * j;
+      if (16 * db >= value_size) continue;
+      bf16x4 v4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[j][qb][i] * inv);
+      *(bf16x4*)(orow + 16 * db + 4 * g) = v4;
+    }
+  }
+}
+
+extern "C" int tnx_latent_gather(const void* latent_pages, const void* rotated_pages, long long latent_stride,
+                                 long long rotated_stride, int page_size, int num_pages, const int* block_table,
+                                 int table_width, const int* row_run, const int* row_pos, void* c_dense, void* r_dense,
+                                 int kv_rank, int rot, int rows, hipStream_t stream) {
+  TNX_REQUIRE(rows >= 0 && kv_rank > 0 && rot >= 0 && page_size > 0 && table_width > 0 && num_pages > 0,
+              "latent_gather: bad sizes");
+  if (rows == 0) return 0;
+  latent_gather_kernel<<<rows, 256, 0, stream>>>((const bf16_t*)latent_pages, (const bf16_t*)rotated_pages,
+                                                 (size_t)latent_stride, (size_t)rotated_stride, page_size, num_pages,
+                                                 block_table, table_width, row_run, row_pos, (bf16_t*)c_dense,
+                                                 (bf16_t*)r_dense, kv_rank, rot);
+  TNX_CHECK_LAUNCH("latent_gather");
+  return 0;
+}
+
+extern "C" int tnx_expanded_attention(const void* q, const void* k_n, const void* k_r, const void* v_t, void* out,
+                                      const int* run_start, const int* cached_lens, const int* ctx_start,
+                                      const int* ctx_base, const int* tile_run, const int* tile_q0, int tiles,
+                                      int tile_tokens, long long rows, const float* freqs, int pairs, float scale,
+                                      int heads, int head_size, int rot, int value_size, int window,
+                                      hipStream_t stream) {
+  TNX_REQUIRE(tiles >= 0 && heads > 0 && head_size > 0 && head_size % 8 == 0 && rot >= 0 && rot % 8 == 0 &&
+                  head_size + rot <= 256 && 2 * pairs <= rot,
+              "expanded_attention: query/key sizes %d + %d", head_size, rot);
+  TNX_REQUIRE(value_size > 0 && value_size % 16 == 0 && value_size <= 256, "expanded_attention: a value of %d elements", value_size);
+  TNX_REQUIRE(tile_tokens == 128 && rows % 64 == 0 && window >= 0, "expanded_attention: tiles of %d queries, %lld rows",
+              tile_tokens, rows);
+  if (tiles == 0) return 0;
+  const int grid = tiles * (tile_tokens / 64) * heads;
+  const int nks = (head_size + rot + 31) / 32, ndv = value_size / 16;
+#define EA_LAUNCH(NKS, NDV)                                                                                          \
+  expanded_attention_kernel<NKS, NDV><<<grid, 256, 0, stream>>>(                                                     \
+      (const bf16_t*)q, (const bf16_t*)k_n, (const bf16_t*)k_r, (const bf16_t*)v_t, (bf16_t*)out, run_start,          \
+      cached_lens, ctx_start, ctx_base, tile_run, tile_q0, tile_tokens, (size_t)rows, freqs, pairs, scale, heads,     \
+      head_size, rot, value_size, window)
+#define EA_VALUES(NKS)                        \
+  if (ndv <= 4) { EA_LAUNCH(NKS, 4); }        \
+  else if (ndv <= 8) { EA_LAUNCH(NKS, 8); }   \
+  else { EA_LAUNCH(NKS, 16); }
+  if (nks <= 2) { EA_VALUES(2) }
+  else if (nks <= 4) { EA_VALUES(4) }
+  else if (nks <= 6) { EA_VALUES(6) }
+  else { EA_VALUES(8) }
+#undef EA_VALUES
+#undef EA_LAUNCH
+  TNX_CHECK_LAUNCH("expanded_attention");
+  return 0;
+}

@@ -106,6 +106,11 @@ _SIGNATURES = {
                                       _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_batched_linear": [_c_void_p, _c_int, _c_ll, _c_ll, _c_void_p, _c_int, _c_void_p, _c_int, _c_float, _c_int,
                                _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_latent_gather": [_c_void_p, _c_void_p, _c_ll, _c_ll, _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p,
+                              _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_expanded_attention": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                                   _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_ll, _c_void_p, _c_int, _c_float,
+                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_latent_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                                      _c_int, _c_int, _c_void_p, _c_void_p, _c_ll, _c_ll, _c_void_p, _c_int, _c_float,
                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -1216,6 +1221,62 @@ class HipOps:
                    _code(w.dtype), _ptr(out), _code(out.dtype), float(alpha), t, heads, n, k, _stream(),
                    work=(f"{t}x{heads}x{n}x{k}", heads * n * k * w.element_size() + t * heads * (k + n) * 2,
                          2.0 * t * heads * n * k))
+        return out
+
+    # Steps that are prompts' runs only, of this many tokens or more: the keys and values of the tokens a run can
+    # see are made from the cached latents once a step (library products) and attention runs on them; a (query,
+    # key) pair then costs 2 (n + r + v) multiply-adds a head instead of the 2 (2 R + r) of the form that reads the
+    # latents as they lie, which is the one for decoding. 0: never.
+    expand_rows = 128
+
+    def latent_expands(self, ctx, head_size, rot, value_size, kv_rank) -> bool:
+        """Whether `latent_attention_expanded` takes this step."""
+        return bool(self.dtype == torch.bfloat16 and self.latent_matrix_unit and self.expand_rows > 0
+                    and ctx.num_tokens >= self.expand_rows and "decode_runs" in ctx.plan
+                    and ctx.plan["decode_runs"].numel() == 0 and head_size % 8 == 0 and rot % 8 == 0
+                    and head_size + rot <= 256 and value_size % 16 == 0 and value_size <= 256 and kv_rank % 8 == 0)
+
+    def latent_attention_expanded(self, q, w_uk, w_uv, num_heads, head_size, rot, value_size, kv_rank, freqs, scale, ctx,
+                                  view, latent_pages, rotated_pages, window=None):
+        """Attention of a step of prompts' runs with expanded keys and values: `[T, H * value_size]`, what
+        `latent_attention` and the product with W_uv give. `w_uk` `[H * head_size, kv_rank]` and `w_uv`
+        `[H * value_size, kv_rank]` are the whole matrices."""
+        t = ctx.num_tokens
+        _want(q, "q", self.dtype, (t, num_heads * (head_size + rot)))
+        num_pages = self._latent_pages(latent_pages, rotated_pages, kv_rank, rot, view.page_size)
+        _want(view.block_table, "block table", torch.int32, (ctx.num_requests, view.width))
+        lens, cached = ctx.run_lens_host.astype(np.int64), ctx.cached_lens_host.astype(np.int64)
+        # what a run can see: from the first key of its first query's window (down to a multiple of 64) to its end,
+        # in dense rows that begin at a multiple of 64
+        base = (np.maximum(0, cached - window + 1) if window else np.zeros_like(cached)) // 64 * 64
+        count = cached + lens - base
+        padded = -(-count // 64) * 64
+        start = np.concatenate([[0], np.cumsum(padded)[:-1]])
+        rows = int(padded.sum())
+        row_run = np.repeat(np.arange(len(lens)), padded)
+        within = np.arange(rows) - np.repeat(start, padded)
+        row_pos = np.where(within < np.repeat(count, padded), np.repeat(base, padded) + within, -1)
+        ints = self.send_ints(np.concatenate([row_run, row_pos, start, base]).astype(np.int32))
+        row_run_d, row_pos_d = ints[:rows], ints[rows:2 * rows]
+        start_d, base_d = ints[2 * rows:2 * rows + len(lens)], ints[2 * rows + len(lens):]
+        c_dense = torch.empty(rows, kv_rank, dtype=self.dtype, device=q.device)
+        r_dense = torch.empty(rows, max(rot, 1), dtype=self.dtype, device=q.device)
+        self._call("latent", "tnx_latent_gather", _ptr(latent_pages), _ptr(rotated_pages), latent_pages.stride(0),
+                   rotated_pages.stride(0), view.page_size, num_pages, _ptr(view.block_table), view.width,
+                   _ptr(row_run_d), _ptr(row_pos_d), _ptr(c_dense), _ptr(r_dense), kv_rank, rot, rows, _stream(),
+                   work=(f"{rows}x{kv_rank}+{rot}", rows * (kv_rank + rot) * 4, 0.0))
+        k_n = self.linear(c_dense, w_uk, None)                                   # [rows, H * n]
+        uv = w_uv.tensor if isinstance(w_uv, PreparedWeight) else w_uv
+        v_t = self.linear(uv, c_dense, None)                                     # [H * v, rows]: tokens side by side
+        out = torch.empty(t, num_heads * value_size, dtype=self.dtype, device=q.device)
+        tiles = ctx.plan["tile_run"].numel()
+        seen = np.minimum(cached + (lens + 1) / 2, window or 1 << 30)
+        self._call("latent", "tnx_expanded_attention", _ptr(q), _ptr(k_n), _ptr(r_dense), _ptr(v_t), _ptr(out),
+                   _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(start_d), _ptr(base_d), _ptr(ctx.plan["tile_run"]),
+                   _ptr(ctx.plan["tile_start"]), tiles, QUERY_TILE, rows, _ptr(freqs), freqs.numel(), float(scale),
+                   num_heads, head_size, rot, value_size, int(window or 0), _stream(),
+                   work=(f"{tiles} tiles", rows * num_heads * (head_size + value_size) * 2.0,
+                         2.0 * num_heads * (head_size + rot + value_size) * float((lens * seen).sum())))
         return out
 
     latent_matrix_unit = True      # tests clear it to run the any-sizes kernel in bfloat16 too

@@ -355,6 +355,40 @@ class ReferenceOps:
             out[s:e] = torch.einsum("hij,jd->ihd", p, c)
         return out.to(self.dtype)
 
+    expand_prompts = False     # tests set it: steps of prompts' runs alone take `latent_attention_expanded`
+
+    def latent_expands(self, ctx, head_size, rot, value_size, kv_rank) -> bool:
+        return bool(self.expand_prompts and int(ctx.run_lens_host.min()) > 1)
+
+    def latent_attention_expanded(self, q, w_uk, w_uv, num_heads, head_size, rot, value_size, kv_rank, freqs, scale, ctx,
+                                  view, latent_pages, rotated_pages, window=None):
+        """Attention with the keys W_uk c and values W_uv c of the cached tokens made explicitly:
+        `[T, H * value_size]`, what `latent_attention` and the product with W_uv give by the other order."""
+        t, ps = q.shape[0], view.page_size
+        out = torch.empty(t, num_heads * value_size, dtype=torch.float32, device=q.device)
+        qh = q.view(t, num_heads, head_size + rot).float()
+        q_r = self._turn(qh[:, :, head_size:], ctx.positions.long(), freqs)
+        starts = ctx.run_start.tolist()
+        for r in range(ctx.num_requests):
+            s, e = starts[r], starts[r + 1]
+            total = int(ctx.cached_lens_host[r]) + (e - s)
+            nb = -(-total // ps)
+            pages = view.block_table[r, :nb].long().clamp(min=0)
+            c = latent_pages[pages].reshape(nb * ps, kv_rank)[:total]
+            c = torch.where(torch.isfinite(c.float()), c.float(), torch.zeros_like(c.float())).to(latent_pages.dtype)
+            k_r = rotated_pages[pages].float().reshape(nb * ps, rot)[:total]
+            k_n = self.linear(c, w_uk).float().view(total, num_heads, head_size)
+            val = self.linear(c, w_uv).float().view(total, num_heads, value_size)
+            scores = (torch.einsum("ihd,jhd->hij", qh[s:e, :, :head_size], k_n) + torch.einsum("ihd,jd->hij", q_r[s:e], k_r)) * scale
+            pos = ctx.positions[s:e].long().unsqueeze(1)
+            j = torch.arange(total, device=q.device).unsqueeze(0)
+            allowed = j <= pos
+            if window is not None:
+                allowed &= pos - j < window
+            p = torch.softmax(scores.masked_fill(~allowed.unsqueeze(0), float("-inf")), dim=-1)
+            out[s:e] = torch.einsum("hij,jhd->ihd", p, val).reshape(e - s, num_heads * value_size)
+        return out.to(self.dtype)
+
     # ---------------------------------------------------------------- output end
 
     def gather_rows(self, x, rows):

@@ -207,6 +207,9 @@ class LatentAttention(Mixer):
         # W_uk a head, transposed: [H, R, n], the matrix that takes a head's q_n to its q_lat
         self.w_uk_t = tensors[uk + s].view(h, self.head_size, self.kv_rank).transpose(1, 2).contiguous()
         self.w_uv = tensors[uv + s].view(h, self.value_size, self.kv_rank).contiguous()
+        # the whole matrices, for steps whose keys and values are made explicitly
+        self.w_uk_whole = ops.prepare_weight(tensors[uk + s])
+        self.w_uv_whole = tensors[uv + s]
         self.w_o = ops.prepare_weight(tensors[o + s])
         self.rotation.load(tensors, prefix + "rotation", ops, dtype)
         self.freqs = self.rotation.frequencies()
@@ -233,6 +236,12 @@ class LatentAttention(Mixer):
         c_q = ops.latent_norms(down, self.q_rank, self.kv_rank if self.own_kv else 0, r if self.own_kv else 0,
                                self.q_norm, self.kv_norm, self.eps, self.freqs, ctx, view, latent, rotated, across)
         q = ops.linear(c_q, self.w_uq, None)
+        if ops.latent_expands(ctx, n, r, self.value_size, self.kv_rank):
+            # a step of prompts' runs alone: keys and values made from the latents, attention on them
+            values = ops.latent_attention_expanded(q, self.w_uk_whole, self.w_uv_whole, heads, n, r, self.value_size,
+                                                   self.kv_rank, self.freqs, self.scale, ctx, view, latent, rotated,
+                                                   self.window)
+            return ops.linear(values, self.w_o, None, residual=residual, out_f32=True, f32_by_library=residual is None)
         q_lat = ops.batched_linear(q.view(-1, heads, n + r)[:, :, :n], self.w_uk_t)
         o_lat = ops.latent_attention(q, q_lat, heads, n, r, self.kv_rank, self.freqs, self.scale, ctx, view,
                                      latent, rotated, across, self.window)
