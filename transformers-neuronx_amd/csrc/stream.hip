@@ -257,8 +257,7 @@ join_norm_conv_kernel(const float* __restrict__ x, const float* __restrict__ y, 
 #pragma unroll
       for (int c = 0; c < PER; ++c) {
         const int k = threadIdx.x + 256 * c;
-        const float* cw = conv_w + (size_t)(4 * min(k, w4 - 1)) * TAPS + j;
-        taps_w[j][c] = (rf4){cw[0], cw[TAPS], cw[2 * TAPS], cw[3 * TAPS]};
+        taps_w[j][c] = ((const rf4*)(conv_w + (size_t)j * width))[min(k, w4 - 1)];
       }
   }
   rf4 kept[KEPT][PER];
@@ -315,8 +314,7 @@ join_norm_conv_kernel(const float* __restrict__ x, const float* __restrict__ y, 
           for (int jj = 1; jj < (TAPS > 0 ? TAPS : 1); ++jj)
             if (jj == j) wj = taps_w[jj][c];
         } else {
-          const float* cw = conv_w + (size_t)(4 * k) * taps + j;
-          wj = (rf4){cw[0], cw[taps], cw[2 * taps], cw[3 * taps]};
+          wj = ((const rf4*)(conv_w + (size_t)j * width))[k];
         }
         acc[c] = acc[c] + wj * v[c];
         if (back == 0) acc[c] = acc[c] + v[c];
@@ -435,8 +433,9 @@ extern "C" int tnx_join_norm_conv(const float* x, const float* y, const float* p
 
 // ------------------------------------------------------------------------------------------------ input convolution
 
-// out[t, d] = h[t, d] + sum_j w[d, j] * h[t - taps + 1 + j, d] over the tokens of t's own request (zeros before
-// its start). Inputs from before the step's run come from the request's state, `[taps, width]`: the input at
+// out[t, d] = h[t, d] + sum_j w[j, d] * h[t - taps + 1 + j, d] over the tokens of t's own request (zeros before
+// its start); the weights come tap by tap, `[taps, width]`, so that a tap's weights of neighbouring channels are
+// neighbours. Inputs from before the step's run come from the request's state, `[taps, width]`: the input at
 // position p lies at place p mod taps. A run's last taps - 1 inputs are written behind the kernel that reads, by
 // another launch; with one place more than is kept, a step of single tokens writes where it does not read, so
 // that running it twice (recorded once, then replayed) reads the same.
@@ -459,7 +458,7 @@ input_conv_kernel(const float* __restrict__ h, const float* __restrict__ w, cons
         x = h[(size_t)(t - back) * width + d];
       else if (back <= p && mine)
         x = mine[(size_t)((p - back) % taps) * width + d];
-      acc += w[(size_t)d * taps + j] * x;
+      acc += w[(size_t)j * width + d] * x;
     }
     store_any(out, out_dtype, (size_t)t * width + d, acc);
   }
@@ -487,8 +486,7 @@ input_conv4_kernel(const float* __restrict__ h, const float* __restrict__ w, con
         x = ((const rf4*)(mine + (size_t)((p - back) % taps) * width))[k];
       else
         continue;
-      const float* cw = w + (size_t)(4 * k) * taps + j;
-      acc = acc + (rf4){cw[0], cw[taps], cw[2 * taps], cw[3 * taps]} * x;
+      acc = acc + ((const rf4*)(w + (size_t)j * width))[k] * x;
     }
     store_chunk(out, out_dtype, (size_t)t * w4 + k, acc);
   }

@@ -266,6 +266,7 @@ class HipOps:
         _code(dtype)
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         self._bias_copies = {}
+        self._conv_copies = {}
         self._later = []
         self._tiles_per_block = {}
         self._landing, self._landing_turn = [None, None], 0
@@ -1083,6 +1084,7 @@ class HipOps:
             return x, self.input_conv(h, conv_w, state, which, ctx, dtype)
         _want(x, "x", torch.float32)
         _want(conv_w, "convolution weights", torch.float32, (width, taps))
+        conv_w = self._taps_first(conv_w)
         mine, stride = None, 0
         if taps > 1:
             _want(state, "convolution state", torch.float32)
@@ -1106,12 +1108,22 @@ class HipOps:
                          t * width * (4 + out.element_size() + (8 if join is not None else 0)), 0.0))
         return (x_out if join is not None else x), out
 
+    def _taps_first(self, weight):
+        """The `[width, taps]` weights of a convolution as the kernels read them, `[taps, width]` (made once a
+        tensor; the original is held with the copy, so that its address names no other tensor meanwhile)."""
+        kept = self._conv_copies.get(weight.data_ptr())
+        if kept is None or kept[0] is not weight:
+            kept = (weight, weight.t().contiguous())
+            self._conv_copies[weight.data_ptr()] = kept
+        return kept[1]
+
     def input_conv(self, h, weight, state, which, ctx, dtype):
         """See `ReferenceOps.input_conv`."""
         _want(h, "h", torch.float32)
         t, width = h.shape
         taps = weight.shape[1]
         _want(weight, "convolution weights", torch.float32, (width, taps))
+        weight = self._taps_first(weight)
         mine, stride = None, 0
         if taps > 1:
             _want(state, "convolution state", torch.float32)
