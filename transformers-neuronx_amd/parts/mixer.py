@@ -141,6 +141,9 @@ class LatentAttention(Mixer):
     score = scale * (q_lat . c + q_r . k_r), and the weighted sum of the c[j] goes through W_uv afterwards.
     c is kept twice, the second time with a page's tokens side by side (`across`), as the other designs'
     values are: the weighted sum contracts over tokens, and the matrix unit wants them next to each other.
+    That order is the one for decoding, where what is read counts. A step of prompts' runs alone may take the
+    other (`ops.latent_expands`): the keys W_uk c and values W_uv c of what the runs can see are made once for
+    the step, and a (query, key) pair costs 2 (n + r + v) multiply-adds a head instead of 2 (2R + r).
 
     `own_kv=False`: no W_dkv; the mixer reads the cache of another call of the run order, whose R, r and
     rotation are its own. `keep`: the tokens the cache keeps: a number, "all", or None for the mixer's own window;
