@@ -1,4 +1,4 @@
-"""An inference engine for decoder-only language models (OPT, Ratesun) on one AMD MI355X."""
+"""An inference engine for decoder-only language models (OPT, Ratesun, Sunatar) on one AMD MI355X."""
 __version__ = "0.1.0"
 
 from .config import ContinuousBatchingConfig, EngineConfig, GenerationConfig, NeuronConfig  # noqa: F401
@@ -13,6 +13,9 @@ def __getattr__(name):
     if name == "RatesunForSampling":
         from .ratesun import model
         return model.RatesunForSampling
+    if name == "SunatarForSampling":
+        from .sunatar import model
+        return model.SunatarForSampling
     if name == "NeuronAutoModelForCausalLM":
         from .modeling_auto import NeuronAutoModelForCausalLM
         return NeuronAutoModelForCausalLM

@@ -40,7 +40,8 @@ _ARCHITECTURES: Dict[str, Architecture] = {}
 # its import before a model folder is read). A program that is started apart (a command line) learns of
 # packages from outside through the environment: TNX_ARCHITECTURE_PACKAGES holds module names, separated
 # by commas, that are importable from where it runs.
-ARCHITECTURE_PACKAGES: List[str] = ["transformers_neuronx_amd.opt", "transformers_neuronx_amd.ratesun"]
+ARCHITECTURE_PACKAGES: List[str] = ["transformers_neuronx_amd.opt", "transformers_neuronx_amd.ratesun",
+                                    "transformers_neuronx_amd.sunatar"]
 PACKAGES_VARIABLE = "TNX_ARCHITECTURE_PACKAGES"
 
 

@@ -51,12 +51,12 @@ class ReferenceOps:
         slots = ctx.slots.long()[ctx.token_request.long()[ctx.logits_rows.long()]]
         kept[slots] = tokens.to(kept.dtype)
 
-    def add_positions(self, src, positions, table, offset, dtype, want_compute):
-        x = src.float() + table[(positions + offset).long()].float()
+    def add_positions(self, src, positions, table, offset, dtype, want_compute, scale=1.0):
+        x = src.float() * scale + table[(positions + offset).long()].float()
         return x, (x.to(dtype) if want_compute else None)
 
-    def to_stream(self, src, dtype, want_compute):
-        x = src.float()
+    def to_stream(self, src, dtype, want_compute, scale=1.0):
+        x = src.float() * scale
         return x, (x.to(dtype) if want_compute else None)
 
     # ---------------------------------------------------------------- norms
@@ -388,6 +388,146 @@ class ReferenceOps:
             p = torch.softmax(scores.masked_fill(~allowed.unsqueeze(0), float("-inf")), dim=-1)
             out[s:e] = torch.einsum("hij,jhd->ihd", p, val).reshape(e - s, num_heads * value_size)
         return out.to(self.dtype)
+
+
+    # ---------------------------------------------------------------- normed, turned and blended projections
+
+    def qkv_prepare(self, proj, num_heads, num_kv, head_size, value_size, cache_head, q_weight, k_weight, eps, freqs,
+                    interleaved, scale, mix_weight, first_values, ctx, view, k_pages, v_pages):
+        """From the float32 projections `proj` `[T, H n + G n + G v]` (bias added) to the queries and the cache:
+        the queries and the keys are each scaled to unit root mean square over their whole width and weighted
+        (`q_weight`, `k_weight`; None: not), the first `2 len(freqs)` elements of every head are turned by
+        position * freqs (pairs (i, i + half), or neighbours with `interleaved`; `freqs` None: not), the queries
+        are multiplied by `scale`, the values become (1 - l) v + l first_values with l = `mix_weight[0]`
+        (`first_values` float32 `[T, G v]`, a view whose rows may lie apart; None: not). Keys and values go to their
+        tokens' places in the pages, heads filled up with zeros to `cache_head` elements; the queries come back
+        `[T, H cache_head]`, filled up alike, in the compute dtype."""
+        t = proj.shape[0]
+        nq, nk, nv = num_heads * head_size, num_kv * head_size, num_kv * value_size
+        x = proj.float()
+        q, k, v = x[:, :nq], x[:, nq:nq + nk], x[:, nq + nk:nq + nk + nv]
+        if q_weight is not None:
+            q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * q_weight.float()
+            k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * k_weight.float()
+        q, k = q.reshape(t, num_heads, head_size), k.reshape(t, num_kv, head_size)
+        if freqs is not None:
+            pos = ctx.positions.long()
+            if interleaved:
+                q, k = self._turn(q, pos, freqs), self._turn(k, pos, freqs)
+            else:
+                half = freqs.numel()
+                angle = pos.float()[:, None, None] * freqs.float()[None, None, :]
+                cos, sin = torch.cos(angle), torch.sin(angle)
+
+                def turned(y):
+                    a, b = y[..., :half], y[..., half:2 * half]
+                    return torch.cat([a * cos - b * sin, b * cos + a * sin, y[..., 2 * half:]], dim=-1)
+                q, k = turned(q), turned(k)
+        if first_values is not None:
+            lam = mix_weight.float()[0]
+            v = (1.0 - lam) * v + lam * first_values.float()
+        v = v.reshape(t, num_kv, value_size)
+        pos = ctx.positions.long()
+        page = view.block_table[ctx.token_request.long(), pos // view.page_size].long()
+        if int(page.min()) < 0:
+            raise RuntimeError("a token of this step has no page")
+        off = pos % view.page_size
+        k_pages[page, :, off, :] = 0
+        k_pages[page, :, off, :head_size] = k.to(k_pages.dtype)
+        v_pages[page, :, :, off] = 0
+        v_pages[page, :, :value_size, off] = v.to(v_pages.dtype)
+        out = torch.zeros(t, num_heads, cache_head, dtype=self.dtype, device=proj.device)
+        out[:, :, :head_size] = (q * scale).to(self.dtype)
+        return out.reshape(t, num_heads * cache_head)
+
+    # ---------------------------------------------------------------- the matrix memory
+
+    def matrix_memory(self, proj, num_heads, head_size, value_size, gate_cap, eps, norm_weight, ctx, memory, normalizer,
+                      peak):
+        """The recurrence of the matrix-memory mixer over a step's runs and what follows it up to the output
+        projection. `proj` float32 `[T, 2 H n + 2 H v + 2 H]`: queries, keys, values, output gates, and a head's
+        input and forget pre-activations (bias added). State float32, in two places by the parity of the
+        position: `memory` `[slots, 2, H, n, v]`, `normalizer` `[slots, 2, H, n]`, `peak` `[slots, 2, H]`; the token
+        at position p reads place (p - 1) & 1 (nothing at p = 0: all zeros) and writes place p & 1. Returns
+        `[T, H v]` in the compute dtype: each head's result at unit root mean square, weighted, times
+        sigmoid(gate)."""
+        t = proj.shape[0]
+        h, n, v = num_heads, head_size, value_size
+        x = proj.float()
+        q = x[:, :h * n].reshape(t, h, n) * (n ** -0.5)
+        k = x[:, h * n:2 * h * n].reshape(t, h, n)
+        val = x[:, 2 * h * n:2 * h * n + h * v].reshape(t, h, v)
+        gate = x[:, 2 * h * n + h * v:2 * h * n + 2 * h * v]
+        gi = gate_cap * torch.tanh(x[:, -2 * h:-h] / gate_cap)
+        gf = torch.nn.functional.logsigmoid(gate_cap * torch.tanh(x[:, -h:] / gate_cap))
+        out = torch.empty(t, h, v, dtype=torch.float32, device=proj.device)
+        start = 0
+        for r in range(ctx.num_requests):
+            count, slot, have = int(ctx.run_lens_host[r]), int(ctx.slots_host[r]), int(ctx.cached_lens_host[r])
+            if have > 0:
+                at = (have - 1) & 1
+                mem, nrm, pk = memory[slot, at].clone(), normalizer[slot, at].clone(), peak[slot, at].clone()
+            else:
+                mem, nrm, pk = torch.zeros_like(memory[slot, 0]), torch.zeros_like(normalizer[slot, 0]), torch.zeros_like(peak[slot, 0])
+            for i in range(start, start + count):
+                new = torch.maximum(gf[i] + pk, gi[i])
+                keep, take = torch.exp(gf[i] + pk - new), torch.exp(gi[i] - new)
+                mem = keep[:, None, None] * mem + take[:, None, None] * (k[i][:, :, None] * val[i][:, None, :])
+                nrm = keep[:, None] * nrm + take[:, None] * k[i]
+                pk = new
+                below = torch.maximum((nrm * q[i]).sum(-1).abs(), torch.exp(-pk)) + 1e-6
+                out[i] = torch.einsum("hnv,hn->hv", mem, q[i]) / below[:, None]
+            at = (have + count - 1) & 1
+            memory[slot, at], normalizer[slot, at], peak[slot, at] = mem, nrm, pk
+            start += count
+        out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps)
+        y = out.reshape(t, h * v) * norm_weight.float() * torch.sigmoid(gate)
+        return y.to(self.dtype)
+
+    # ---------------------------------------------------------------- experts
+
+    def route(self, z, top, score="sigmoid", renormalize=False):
+        """float32 router logits `[T, E]` -> (int32 `[T, top]` the experts with the largest scores, the lower
+        number first where two are equal; float32 `[T, top]` their scores, sigmoid(z) or softmax(z), divided by
+        their sum with `renormalize`)."""
+        s = torch.sigmoid(z.float()) if score == "sigmoid" else torch.softmax(z.float(), dim=-1)
+        order = torch.sort(s, dim=-1, descending=True, stable=True).indices[:, :top]
+        w = torch.gather(s, 1, order)
+        if renormalize:
+            w = w / w.sum(-1, keepdim=True)
+        return order.to(torch.int32).contiguous(), w.contiguous()
+
+    @staticmethod
+    def _gate(g, activation):
+        if activation == "silu":
+            return g * torch.sigmoid(g)
+        return ReferenceOps.activation(g, activation)
+
+    def gated_activation(self, gate_up, activation, weights=None):
+        """`act(g) * u` from float32 `[T, 2 F]` = [g | u], in the compute dtype."""
+        f = gate_up.shape[1] // 2
+        g, u = gate_up[:, :f].float(), gate_up[:, f:].float()
+        return (self._gate(g, activation) * u).to(self.dtype)
+
+    def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None):
+        """float32 `residual + sum_c expert_(chosen[t, c])(h[t])` with the weights `weights[t, c]` on the expert's
+        input (`weight_on="input"`: act(w g) * (w u), the float32 sums of the first product times w) or on its
+        output. `w_gate_up` `[E, 2 F, D]` (gate rows, then up rows), `w_down` `[E, D, F]`."""
+        t, top = chosen.shape
+        f = w_down.shape[2]
+        out = residual.float().clone() if residual is not None else torch.zeros(t, w_down.shape[1], dtype=torch.float32,
+                                                                                device=h.device)
+        x = h.to(w_gate_up.dtype).float()
+        for c in range(top):
+            e = chosen[:, c].long()
+            gu = torch.einsum("tk,tnk->tn", x, w_gate_up[e].float())
+            w = weights[:, c].float()[:, None]
+            if weight_on == "input":
+                gu = gu * w
+            inner = (self._gate(gu[:, :f], activation) * gu[:, f:]).to(self.dtype)
+            y = torch.einsum("tf,tdf->td", inner.to(w_down.dtype).float(), w_down[e].float())
+            out = out + (y if weight_on == "input" else y * w)
+        return out
 
     # ---------------------------------------------------------------- output end
 

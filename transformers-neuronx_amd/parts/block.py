@@ -51,6 +51,19 @@ class PostNormBlock(Block):
         return Stream(x, h)
 
 
+@register_block("parallel")
+class ParallelBlock(Block):
+    """`h = norm(x)`, `x = x + mixer(h) + feed_forward(h)`: one norm, and both parts read its output. The sum
+    is float32: the mixer's last product adds the stream, the feed-forward's adds that."""
+
+    recordable = True
+
+    def forward(self, stream: Stream, ctx, cache) -> Stream:
+        h = self.mixer_norm.forward(stream.x, False, True)[1]
+        x = debug.tap("after_mixer", self.mixer.forward(h, ctx, cache, stream.x))
+        return Stream(self.feed_forward.forward(h, ctx, x), None)
+
+
 @register_block("sandwich")
 class SandwichBlock(Block):
     """A norm before and after each part, the part's normed result scaled before it joins the stream:

@@ -17,8 +17,10 @@ class TokenEmbedding(Part):
     recordable = True
 
     def __init__(self, vocab: int, embed_width: int, width: int, position: PartSpec,
-                 table_name: str, projection_name: Optional[str], position_name: str):
+                 table_name: str, projection_name: Optional[str], position_name: str, scale: float = 1.0):
+        """`scale`: the token's row times this number (in float32, where the row joins the stream)."""
         self.vocab, self.embed_width, self.width = vocab, embed_width, width
+        self.scale = float(scale)
         self.table_name, self.projection_name, self.position_name = table_name, projection_name, position_name
         self.position = POSITIONS.build(position)
         self.projects = embed_width != width
@@ -39,7 +41,10 @@ class TokenEmbedding(Part):
         x = self.ops.embed(ctx.token_ids, self.table, self.dtype, ctx.kept_tokens)
         if self.projects:
             x = self.ops.linear(x, self.projection, None)
-        xf, xc = self.position.at_input(x, ctx.positions, want_compute)
+        if self.scale != 1.0:
+            xf, xc = self.position.at_input(x, ctx.positions, want_compute, scale=self.scale)
+        else:
+            xf, xc = self.position.at_input(x, ctx.positions, want_compute)
         return Stream(xf, xc)
 
 

@@ -69,3 +69,75 @@ class NoFeedForward(FeedForward):
 
     def forward(self, h, ctx, residual):
         return residual
+
+
+@register_feed_forward("mixture")
+class ExpertMixture(FeedForward):
+    """A mixture of gated experts, of which a token takes `top`, and optionally one more that every token takes.
+
+    Router: z = W_r h in float32, scores s = sigmoid(z) (`score="sigmoid"`) or softmax(z) (`"softmax"`); a token's
+    experts are the `top` with the largest scores (the lower number where two are equal), their weights the
+    scores, divided by their sum with `renormalize`. An expert is W_down (act(W_gate x) * (W_up x)), no biases.
+    `weight_on="input"`: the result is the sum of expert(w h), the weight applied to what the expert reads;
+    `"output"`: the sum of w expert(h). The shared expert (`shared_inner` > 0) is of the same form, reads h and
+    is added. The weights enter the float32 sums of the first products, so nothing is rounded twice."""
+
+    recordable = True
+
+    def __init__(self, width: int, experts: int, top: int, inner: int, router_name: str, expert_name: str, names,
+                 shared_inner: int = 0, shared_name: str = "shared.", score: str = "sigmoid", renormalize: bool = False,
+                 weight_on: str = "output", activation: str = "silu", weight_suffix: str = ""):
+        """`expert_name`: a format string that takes the expert's number ("e{}."); `names`: the names of an
+        expert's gate, up and down matrices."""
+        if not 1 <= top <= experts:
+            raise ValueError(f"a token takes {top} of {experts} experts")
+        if score not in ("sigmoid", "softmax") or weight_on not in ("input", "output") or activation not in ("silu", "gelu_new"):
+            raise ValueError(f"mixture: score {score!r}, weight_on {weight_on!r}, activation {activation!r}")
+        self.width, self.experts, self.top, self.inner, self.shared_inner = width, experts, top, inner, shared_inner
+        self.router_name, self.expert_name, self.shared_name = router_name, expert_name, shared_name
+        self.names, self.weight_suffix = tuple(names), weight_suffix
+        self.score, self.renormalize, self.weight_on, self.activation = score, bool(renormalize), weight_on, activation
+
+    def _expert_decls(self, prefix: str, inner: int) -> List[ParamDecl]:
+        g, u, d = self.names
+        s = self.weight_suffix
+        return [ParamDecl(f"{prefix}{g}{s}", (inner, self.width)), ParamDecl(f"{prefix}{u}{s}", (inner, self.width)),
+                ParamDecl(f"{prefix}{d}{s}", (self.width, inner))]
+
+    def param_decls(self, prefix: str) -> List[ParamDecl]:
+        d = []
+        for e in range(self.experts):
+            d += self._expert_decls(prefix + self.expert_name.format(e), self.inner)
+        d.append(ParamDecl(f"{prefix}{self.router_name}{self.weight_suffix}", (self.experts, self.width)))
+        if self.shared_inner:
+            d += self._expert_decls(prefix + self.shared_name, self.shared_inner)
+        return d
+
+    def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
+        import torch
+        super().load(tensors, prefix, ops, dtype)
+        g, u, d = self.names
+        s = self.weight_suffix
+        each = [prefix + self.expert_name.format(e) for e in range(self.experts)]
+        # an expert's gate rows, then its up rows: `[experts, 2 inner, width]`; the down matrices `[experts, width, inner]`
+        self.w_gate_up = torch.stack([torch.cat([tensors[f"{p}{g}{s}"], tensors[f"{p}{u}{s}"]], dim=0) for p in each]).contiguous()
+        self.w_down = torch.stack([tensors[f"{p}{d}{s}"] for p in each]).contiguous()
+        self.w_router = ops.prepare_weight(tensors[f"{prefix}{self.router_name}{s}"])
+        if self.shared_inner:
+            p = prefix + self.shared_name
+            self.w_shared_in = ops.prepare_weight(torch.cat([tensors[f"{p}{g}{s}"], tensors[f"{p}{u}{s}"]], dim=0).contiguous())
+            self.w_shared_down = ops.prepare_weight(tensors[f"{p}{d}{s}"])
+
+    def flops_per_token(self, keys: float = 0.0) -> float:
+        return 2.0 * self.width * (self.experts + 3 * self.top * self.inner + 3 * self.shared_inner)
+
+    def forward(self, h, ctx, residual):
+        ops = self.ops
+        z = ops.linear(h, self.w_router, None, out_f32=True)
+        chosen, weights = ops.route(z, self.top, self.score, self.renormalize)
+        x = ops.expert_mixture(h, chosen, weights, self.w_gate_up, self.w_down, self.activation, self.weight_on, residual)
+        if not self.shared_inner:
+            return x
+        inner = ops.gated_activation(ops.linear(h, self.w_shared_in, None, out_f32=True, f32_by_library=True),
+                                     self.activation)
+        return ops.linear(inner, self.w_shared_down, None, residual=x, out_f32=True)

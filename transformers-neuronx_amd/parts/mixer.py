@@ -32,40 +32,76 @@ class Attention(Mixer):
 
     def __init__(self, width: int, num_heads: int, head_size: int, names, num_kv_heads: Optional[int] = None,
                  bias: bool = True, window: Optional[int] = None, scale: Optional[float] = None,
-                 own_kv: bool = True, rotation=None):
+                 own_kv: bool = True, rotation=None, value_size: Optional[int] = None, out_bias: Optional[bool] = None,
+                 qk_norm=None, value_mix=None, weight_suffix: str = ".weight", bias_suffix: str = ".bias"):
         """`names`: the checkpoint's names of the query, key, value and output projections, relative to
-        the mixer's prefix (the architecture's spec gives them)."""
+        the mixer's prefix (the architecture's spec gives them); a matrix's name adds `weight_suffix`, a bias's
+        `bias_suffix`. `out_bias`: whether the output projection has a bias (as the others, if not said).
+
+        `value_size`: elements of a value head where they differ from a query/key head's `head_size`.
+        `qk_norm` = {eps, suffix}: queries and keys are scaled to unit root mean square over the whole
+        projection, all heads at once, and weighted (the tensors `<query name><suffix>`, `<key name><suffix>`),
+        after the bias and before the rotation. `value_mix` = {key, first, name}: the layers that give the same
+        `key` blend their values with those the `first` of them made for the same token,
+        v = (1 - l) v + l v_first with l the scalar tensor `name`; the blended values are what is cached. The
+        first blends nothing and has no such tensor. A rotation whose pairs are not neighbours
+        (`interleaved=False`) hands its frequencies to the kernel that norms, turns and stores.
+        These take the float32 route: the projection's float32 result goes through one kernel (`ops.qkv_prepare`)
+        that norms, turns, scales, blends and stores, and heads of unequal sizes are cached filled up with
+        zeros to one size, a multiple of 16."""
         self.width, self.num_heads, self.head_size = width, num_heads, head_size
         self.num_kv_heads = num_kv_heads if num_kv_heads is not None else num_heads
         if self.num_heads % self.num_kv_heads:
             raise ValueError(f"num_heads ({num_heads}) must be a multiple of num_kv_heads ({self.num_kv_heads})")
-        if head_size % 16 or not 16 <= head_size <= 256:
+        self.value_size = value_size if value_size is not None else head_size
+        self.qk_norm = dict(qk_norm) if qk_norm else None
+        self.value_mix = dict(value_mix) if value_mix else None
+        self.rotation = POSITIONS.build(rotation) if rotation is not None else None
+        halves = self.rotation is not None and not getattr(self.rotation, "interleaved", True)
+        self.prepared = bool(self.qk_norm or self.value_mix or halves or self.value_size != head_size)
+        if self.prepared:
+            if not own_kv:
+                raise ValueError("a mixer that norms, blends or fills up its heads makes its own keys and values")
+            if self.rotation is not None and not hasattr(self.rotation, "frequencies"):
+                raise ValueError("the float32 route turns by a rotation that gives `frequencies()`")
+            self.cache_head = -(-max(head_size, self.value_size) // 16) * 16
+        else:
+            self.cache_head = head_size
+        if self.cache_head % 16 or not 16 <= self.cache_head <= 256:
             raise ValueError(f"head_size must be a multiple of 16 between 16 and 256, got {head_size}")
         self.has_bias, self.window, self.own_kv = bias, window, own_kv
+        self.has_out_bias = bias if out_bias is None else bool(out_bias)
+        self.weight_suffix, self.bias_suffix = weight_suffix, bias_suffix
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_size)
         self.names = tuple(names)
-        self.rotation = POSITIONS.build(rotation) if rotation is not None else None
         if self.rotation is not None and not getattr(self.rotation, "recordable", False):
             self.recordable = False
         if len(self.names) != 4:
             raise ValueError("names: the query, key, value and output projections, four names")
 
     def cache_need(self) -> Optional[CacheNeed]:
-        return CacheNeed("paged", kv_heads=self.num_kv_heads, head_size=self.head_size, window=self.window)
+        return CacheNeed("paged", kv_heads=self.num_kv_heads, head_size=self.cache_head, window=self.window)
 
     def param_decls(self, prefix: str) -> List[ParamDecl]:
         qn, kn, vn, on = self.names
+        ws, bs = self.weight_suffix, self.bias_suffix
         q_out = self.num_heads * self.head_size
         kv_out = self.num_kv_heads * self.head_size
-        outs = [(qn, q_out)] + ([(kn, kv_out), (vn, kv_out)] if self.own_kv else [])
+        v_out = self.num_kv_heads * self.value_size
+        outs = [(qn, q_out)] + ([(kn, kv_out), (vn, v_out)] if self.own_kv else [])
         d = []
         for n, out in outs:
-            d.append(ParamDecl(f"{prefix}{n}.weight", (out, self.width)))
+            d.append(ParamDecl(f"{prefix}{n}{ws}", (out, self.width)))
             if self.has_bias:
-                d.append(ParamDecl(f"{prefix}{n}.bias", (out,), "vector"))
-        d.append(ParamDecl(f"{prefix}{on}.weight", (self.width, q_out)))
-        if self.has_bias:
-            d.append(ParamDecl(f"{prefix}{on}.bias", (self.width,), "vector"))
+                d.append(ParamDecl(f"{prefix}{n}{bs}", (out,), "vector"))
+        d.append(ParamDecl(f"{prefix}{on}{ws}", (self.width, self.num_heads * self.value_size)))
+        if self.has_out_bias:
+            d.append(ParamDecl(f"{prefix}{on}{bs}", (self.width,), "vector"))
+        if self.qk_norm:
+            d += [ParamDecl(f"{prefix}{qn}{self.qk_norm['suffix']}", (q_out,), "vector", "around_one"),
+                  ParamDecl(f"{prefix}{kn}{self.qk_norm['suffix']}", (kv_out,), "vector", "around_one")]
+        if self.value_mix and not self.value_mix["first"]:
+            d.append(ParamDecl(f"{prefix}{self.value_mix['name']}", (), "vector", "around_half"))
         if self.rotation is not None:
             d += self.rotation.param_decls(prefix + "rotation")
         return d
@@ -73,21 +109,37 @@ class Attention(Mixer):
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
         super().load(tensors, prefix, ops, dtype)
         qn, kn, vn, on = self.names
+        ws, bs = self.weight_suffix, self.bias_suffix
         ins = [qn] + ([kn, vn] if self.own_kv else [])
         # One fused projection: a plain concatenation of the rows (the reference's
         # fused form interleaves per tensor-parallel shard, utils.py:189-242).
-        self.w_qkv = ops.prepare_weight(torch.cat([tensors[f"{prefix}{n}.weight"] for n in ins], dim=0).contiguous())
-        self.b_qkv = (torch.cat([tensors[f"{prefix}{n}.bias"] for n in ins], dim=0).contiguous()
+        self.w_qkv = ops.prepare_weight(torch.cat([tensors[f"{prefix}{n}{ws}"] for n in ins], dim=0).contiguous())
+        self.b_qkv = (torch.cat([tensors[f"{prefix}{n}{bs}"] for n in ins], dim=0).contiguous()
                       if self.has_bias else None)
-        self.w_out = ops.prepare_weight(tensors[f"{prefix}{on}.weight"])
-        self.b_out = tensors[f"{prefix}{on}.bias"] if self.has_bias else None
+        w_out = tensors[f"{prefix}{on}{ws}"]
+        if self.cache_head != self.value_size:
+            # the attention's result has heads of the cache's size: the columns that meet the filling are zeros
+            wide = w_out.new_zeros(self.width, self.num_heads, self.cache_head)
+            wide[:, :, :self.value_size] = w_out.view(self.width, self.num_heads, self.value_size)
+            w_out = wide.view(self.width, self.num_heads * self.cache_head).contiguous()
+        self.w_out = ops.prepare_weight(w_out)
+        self.b_out = tensors[f"{prefix}{on}{bs}"] if self.has_out_bias else None
         self.turn = None
+        self.q_norm = self.k_norm = self.mix_weight = self.freqs = None
         if self.rotation is not None:
             self.rotation.load(tensors, prefix + "rotation", ops, dtype)
-            self.turn = self.rotation.pair_tables(self.head_size)     # the pairwise form: applied by the projection
+            if self.prepared:
+                self.freqs = self.rotation.frequencies()
+            else:
+                self.turn = self.rotation.pair_tables(self.head_size)     # the pairwise form: applied by the projection
+        if self.qk_norm:
+            self.q_norm = tensors[f"{prefix}{qn}{self.qk_norm['suffix']}"]
+            self.k_norm = tensors[f"{prefix}{kn}{self.qk_norm['suffix']}"]
+        if self.value_mix and not self.value_mix["first"]:
+            self.mix_weight = tensors[f"{prefix}{self.value_mix['name']}"].reshape(1)
 
     def first_weight(self):
-        return self.w_qkv
+        return None if self.prepared else self.w_qkv
 
     def step_planners(self):
         from ..kernels.attention_plan import attention_plan
@@ -95,16 +147,43 @@ class Attention(Mixer):
 
     def launch_shape(self, step):
         shape = getattr(self.ops, "attention_launch_shape", None)
-        return shape(step, self.num_heads, self.window, self.head_size, self.num_kv_heads) if shape is not None else None
+        return shape(step, self.num_heads, self.window, self.cache_head, self.num_kv_heads) if shape is not None else None
 
     def flops_per_token(self, keys: float = 0.0) -> float:
         seen = min(keys, self.window) if self.window else keys
-        return super().flops_per_token(keys) + 4.0 * self.num_heads * self.head_size * seen   # q k^T and p v
+        # q k^T and p v
+        return super().flops_per_token(keys) + 2.0 * self.num_heads * (self.head_size + self.value_size) * seen
+
+    def _forward_prepared(self, h, ctx, cache, residual, view):
+        """The float32 route: projection with its bias, one kernel that norms, turns, scales, blends and stores,
+        attention over heads of the cache's size, the output projection."""
+        ops = self.ops
+        proj = ops.linear(h, self.w_qkv, self.b_qkv, out_f32=True, f32_by_library=True)
+        first = None
+        if self.value_mix:
+            key = ("value mix", self.value_mix["key"])
+            if self.value_mix["first"]:
+                # what the later layers blend with: this step's values as this layer made them
+                ctx.memo[key] = proj[:, (self.num_heads + self.num_kv_heads) * self.head_size:]
+            else:
+                first = ctx.memo.get(key)
+                if first is None:
+                    raise ValueError("a layer blends its values with those of a layer that has not run in this pass")
+        rot = self.rotation
+        q = ops.qkv_prepare(proj, self.num_heads, self.num_kv_heads, self.head_size, self.value_size, self.cache_head,
+                            self.q_norm, self.k_norm, self.qk_norm["eps"] if self.qk_norm else 0.0, self.freqs,
+                            bool(rot.interleaved) if rot is not None else False, self.scale, self.mix_weight, first,
+                            ctx, view, cache.k_pages, cache.v_pages)
+        c = ops.attention(q, self.num_heads, self.num_kv_heads, self.cache_head, ctx, view, cache.k_pages,
+                          cache.v_pages, self.window)
+        return ops.linear(c, self.w_out, self.b_out, residual=residual, out_f32=True)
 
     def forward(self, h, ctx, cache, residual):
         if cache.writes != self.own_kv:
             raise ValueError("an attention mixer with own_kv writes its cache; one without reads another's")
         view = ctx.groups[cache.group]
+        if self.prepared:
+            return self._forward_prepared(h, ctx, cache, residual, view)
         kv_write = self.num_kv_heads if self.own_kv else 0
         if self.rotation is not None and self.turn is None:
             # the projections with their bias, turned by the encoding, then scaled and stored
@@ -251,3 +330,81 @@ class LatentAttention(Mixer):
         values = ops.batched_linear(o_lat, self.w_uv)
         return ops.linear(values.view(-1, heads * self.value_size), self.w_o, None, residual=residual, out_f32=True,
                           f32_by_library=residual is None)
+
+
+@register_mixer("mlstm")
+class MatrixMemory(Mixer):
+    """A matrix memory a head that is carried from token to token (the mLSTM cell of xLSTM): no cache that grows,
+    a state of fixed size a request.
+
+    With H heads, n query/key and v value elements a head, for the token at step t:
+        q = W_q h / sqrt(n),  k = W_k h,  val = W_v h
+        i = cap tanh((W_i h + b_i) / cap),  f = logsigmoid(cap tanh((W_f h + b_f) / cap))        (a number a head each)
+        m_t = max(f + m_(t-1), i)
+        S_t = exp(f + m_(t-1) - m_t) S_(t-1) + exp(i - m_t) k val^T,   n_t likewise with k alone
+        o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + 1e-6)
+    S, n and m start at zero. Each head's o is scaled to unit root mean square, the heads side by side are
+    weighted by `norm`, multiplied by sigmoid(W_g h), and W_o follows. Gates, state and norms are float32.
+
+    The state is kept in two places by the parity of the position: the token at position p reads place
+    (p - 1) & 1 and writes place p & 1, so that a step of single tokens that is run again reads what it read the
+    first time. Position 0 reads nothing.
+    """
+
+    recordable = True
+
+    def __init__(self, width: int, num_heads: int, head_size: int, value_size: int, gate_cap: float, eps: float, names,
+                 weight_suffix: str = "", bias_suffix: str = ".b"):
+        """`names`: the checkpoint's names, relative to the mixer's prefix, of W_q, W_k, W_v, W_g, W_o, W_i, W_f
+        (the two gates have a bias, their name with `bias_suffix`) and of the weight of the norm after the cell."""
+        self.width, self.num_heads, self.head_size, self.value_size = width, num_heads, head_size, value_size
+        self.gate_cap, self.eps = float(gate_cap), float(eps)
+        self.names = tuple(names)
+        if len(self.names) != 8:
+            raise ValueError("names: W_q, W_k, W_v, W_g, W_o, W_i, W_f and the norm, eight names")
+        self.weight_suffix, self.bias_suffix = weight_suffix, bias_suffix
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        h, n, v = self.num_heads, self.head_size, self.value_size
+        return CacheNeed("state", state_shapes=(("memory", (2, h, n, v)), ("normalizer", (2, h, n)), ("peak", (2, h))))
+
+    def _rows(self):
+        h, n, v = self.num_heads, self.head_size, self.value_size
+        q, k, val, g, o, i, f, norm = self.names
+        return [(q, h * n), (k, h * n), (val, h * v), (g, h * v), (i, h), (f, h)]
+
+    def param_decls(self, prefix: str) -> List[ParamDecl]:
+        ws, bs = self.weight_suffix, self.bias_suffix
+        q, k, val, g, o, i, f, norm = self.names
+        d = [ParamDecl(f"{prefix}{name}{ws}", (rows, self.width)) for name, rows in self._rows()]
+        d += [ParamDecl(f"{prefix}{i}{bs}", (self.num_heads,), "vector"),
+              ParamDecl(f"{prefix}{f}{bs}", (self.num_heads,), "vector"),
+              ParamDecl(f"{prefix}{o}{ws}", (self.width, self.num_heads * self.value_size)),
+              ParamDecl(f"{prefix}{norm}", (self.num_heads * self.value_size,), "vector", "around_one")]
+        return d
+
+    def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
+        super().load(tensors, prefix, ops, dtype)
+        ws, bs = self.weight_suffix, self.bias_suffix
+        q, k, val, g, o, i, f, norm = self.names
+        # one product for everything the cell reads: the rows of W_q, W_k, W_v, W_g, W_i, W_f
+        self.w_in = ops.prepare_weight(torch.cat([tensors[f"{prefix}{name}{ws}"] for name, _ in self._rows()], dim=0)
+                                       .contiguous())
+        gates = torch.cat([tensors[f"{prefix}{i}{bs}"], tensors[f"{prefix}{f}{bs}"]])
+        bias = gates.new_zeros(self.w_in.shape[0])
+        bias[-2 * self.num_heads:] = gates
+        self.b_in = bias.contiguous()
+        self.w_out = ops.prepare_weight(tensors[f"{prefix}{o}{ws}"])
+        self.norm_weight = tensors[f"{prefix}{norm}"]
+
+    def flops_per_token(self, keys: float = 0.0) -> float:
+        # the memory's update and its product with the query, a head
+        return super().flops_per_token(keys) + 4.0 * self.num_heads * self.head_size * self.value_size
+
+    def forward(self, h, ctx, cache, residual):
+        ops = self.ops
+        proj = ops.linear(h, self.w_in, self.b_in, out_f32=True, f32_by_library=True)
+        st = cache.state
+        y = ops.matrix_memory(proj, self.num_heads, self.head_size, self.value_size, self.gate_cap, self.eps,
+                              self.norm_weight, ctx, st["memory"], st["normalizer"], st["peak"])
+        return ops.linear(y, self.w_out, None, residual=residual, out_f32=True)

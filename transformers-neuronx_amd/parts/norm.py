@@ -14,23 +14,27 @@ class LayerNorm(Norm):
     recordable = True
 
     def __init__(self, width: int, eps: float, affine: bool = True, weight_suffix: str = ".weight",
-                 bias_suffix: str = ".bias"):
-        """`weight_suffix`, `bias_suffix`: what the checkpoint's names of the two vectors add to the norm's."""
+                 bias_suffix: str = ".bias", bias: bool = True):
+        """`weight_suffix`, `bias_suffix`: what the checkpoint's names of the two vectors add to the norm's;
+        `bias=False`: an affine norm with a weight alone."""
         self.width, self.eps, self.affine = width, float(eps), affine
+        self.has_bias = bool(bias) and affine
         self.weight_suffix, self.bias_suffix = weight_suffix, bias_suffix
         self.weight = self.bias = None
 
     def param_decls(self, prefix: str) -> List[ParamDecl]:
         if not self.affine:
             return []
-        return [ParamDecl(prefix + self.weight_suffix, (self.width,), "vector", "around_one"),
-                ParamDecl(prefix + self.bias_suffix, (self.width,), "vector", "normal")]
+        d = [ParamDecl(prefix + self.weight_suffix, (self.width,), "vector", "around_one")]
+        if self.has_bias:
+            d.append(ParamDecl(prefix + self.bias_suffix, (self.width,), "vector", "normal"))
+        return d
 
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
         super().load(tensors, prefix, ops, dtype)
         if self.affine:
             self.weight = tensors[prefix + self.weight_suffix]
-            self.bias = tensors[prefix + self.bias_suffix]
+            self.bias = tensors[prefix + self.bias_suffix] if self.has_bias else None
 
     def forward(self, x, want_f32: bool, want_compute: bool):
         return self.ops.layernorm(x, self.weight, self.bias, self.eps, self.dtype, want_f32, want_compute)

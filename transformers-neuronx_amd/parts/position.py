@@ -24,9 +24,10 @@ class LearnedPositions(PositionEncoding):
         super().load(tensors, prefix, ops, dtype)
         self.table = tensors[prefix + ".weight"]
 
-    def at_input(self, x, positions, want_compute: bool):
-        """x `[T, width]` (any float dtype) -> (float32 sum, compute-dtype copy or None)."""
-        return self.ops.add_positions(x, positions, self.table, self.offset, self.dtype, want_compute)
+    def at_input(self, x, positions, want_compute: bool, scale: float = 1.0):
+        """x `[T, width]` (any float dtype) -> (float32 sum, compute-dtype copy or None); `scale` multiplies the
+        token's row before the position's joins it."""
+        return self.ops.add_positions(x, positions, self.table, self.offset, self.dtype, want_compute, scale=scale)
 
 
 @register_position("none")
@@ -38,8 +39,8 @@ class NoPositions(PositionEncoding):
     def __init__(self, **_):
         pass
 
-    def at_input(self, x, positions, want_compute: bool):
-        return self.ops.to_stream(x, self.dtype, want_compute)
+    def at_input(self, x, positions, want_compute: bool, scale: float = 1.0):
+        return self.ops.to_stream(x, self.dtype, want_compute, scale=scale)
 
 
 @register_position("rotary")
@@ -49,15 +50,26 @@ class RotaryPositions(PositionEncoding):
     pair (u, v) at position p becomes (u cos a - v sin a, v cos a + u sin a), a = p * base^(-2i / dims). The
     elements beyond `dims` pass. Positions, frequencies and angles are float32.
 
+    `scaling` = {factor, low, high, original} stretches the slow turns for requests longer than `original`
+    tokens: a frequency f with wavelength l = 2 pi / f is kept where l < original / high, becomes f / factor
+    where l > original / low, and between the two (1 - s) f / factor + s f with
+    s = (original / l - low) / (high - low).
+
     Two ways to use it: `pair_tables` (the attention mixer's pairwise form, for `max_positions` positions,
     interleaved pairs only), or `frequencies()`, for a mixer whose kernels make the angles themselves."""
 
     recordable = True
 
-    def __init__(self, base: float, dims: int, max_positions: int = 0, interleaved: bool = True):
+    def __init__(self, base: float, dims: int, max_positions: int = 0, interleaved: bool = True, scaling=None):
         if dims % 2 or dims < 0:
             raise ValueError(f"rotary positions turn pairs: dims must be even, got {dims}")
         self.base, self.dims, self.max_positions, self.interleaved = float(base), dims, max_positions, interleaved
+        self.scaling = dict(scaling) if scaling else None
+        if self.scaling:
+            missing = [k for k in ("factor", "low", "high", "original") if k not in self.scaling]
+            if missing or self.scaling["high"] == self.scaling["low"]:
+                raise ValueError(f"scaling of rotary frequencies: factor, low, high (other than low) and original; "
+                                 f"got {self.scaling!r}")
         self.device = "cpu"
 
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
@@ -70,7 +82,15 @@ class RotaryPositions(PositionEncoding):
         if getattr(self, "_freqs", None) is None:
             import torch
             i = torch.arange(self.dims // 2, dtype=torch.float64)
-            self._freqs = (self.base ** (-2.0 * i / max(self.dims, 1))).to(torch.float32).to(self.device)
+            f = self.base ** (-2.0 * i / max(self.dims, 1))
+            if self.scaling:
+                import math
+                c = self.scaling
+                turns = float(c["original"]) * f / (2.0 * math.pi)        # original / wavelength
+                s = (turns - c["low"]) / (c["high"] - c["low"])
+                blend = (1.0 - s) * f / c["factor"] + s * f
+                f = torch.where(turns > c["high"], f, torch.where(turns < c["low"], f / c["factor"], blend))
+            self._freqs = f.to(torch.float32).to(self.device)
         return self._freqs
 
     def pair_tables(self, head_size: int):

@@ -28,7 +28,7 @@ class ParamDecl:
             'vector' (bias or norm parameter, kept in float32),
             'index' (integer table, kept in int32)
     init    how the random-weights mode draws it: 'normal' (mean 0),
-            'around_one' (mean 1), 'around_mean' (mean 1 / its size), all with the configuration's deviation
+            'around_one' (mean 1), 'around_half' (mean 1/2), 'around_mean' (mean 1 / its size), all with the configuration's deviation
     tied_to another tensor's name that stands in when this one is absent
     """
     name: str

@@ -36,6 +36,8 @@ def random_tensors(decls: List[ParamDecl], std: float, seed: int, matrix_dtype: 
         t = torch.randn(d.shape, generator=gen, device=device, dtype=torch.float32) * std
         if d.init == "around_one":
             t += 1.0
+        elif d.init == "around_half":      # a blending weight: somewhere about the middle between 0 and 1
+            t += 0.5
         elif d.init == "around_mean":      # weights of an average: about 1 / their number each
             t += 1.0 / max(1, t.numel())
         out[d.name] = t if d.role == "vector" else t.to(matrix_dtype)
