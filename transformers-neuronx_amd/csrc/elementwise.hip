@@ -62,13 +62,14 @@ extern "C" int tnx_device_pointer(void* host, void** device) {
 // x[t, :] = src[t, :] + table[positions[t] + offset, :] in float32; a copy in `cd_dtype` beside it.
 __global__ void add_positions_kernel(const void* __restrict__ src, int src_dtype, const int* __restrict__ positions,
                                      const void* __restrict__ table, int table_dtype, int table_rows, int offset,
-                                     float* __restrict__ out_f32, void* __restrict__ out_cd, int cd_dtype, int width) {
+                                     float* __restrict__ out_f32, void* __restrict__ out_cd, int cd_dtype, int width,
+                                     float scale) {
   const int t = blockIdx.x;
   size_t base = (size_t)t * width;
   int row = table ? positions[t] + offset : 0;
   if (table && (row < 0 || row >= table_rows)) row = 0;  // the host checks positions
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    float v = load_any(src, src_dtype, base + i);
+    float v = load_any(src, src_dtype, base + i) * scale;   // the token's row times `scale`, in float32
     if (table) v += load_any(table, table_dtype, (size_t)row * width + i);
     out_f32[base + i] = v;
     if (out_cd) store_any(out_cd, cd_dtype, base + i, v);
@@ -77,11 +78,11 @@ __global__ void add_positions_kernel(const void* __restrict__ src, int src_dtype
 
 extern "C" int tnx_add_positions(const void* src, int src_dtype, const int* positions, const void* table,
                                  int table_dtype, int table_rows, int offset, float* out_f32, void* out_cd,
-                                 int cd_dtype, int tokens, int width, hipStream_t stream) {
+                                 int cd_dtype, int tokens, int width, float scale, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && width > 0, "add_positions: bad sizes tokens=%d width=%d", tokens, width);
   if (tokens == 0) return 0;
   add_positions_kernel<<<tokens, 256, 0, stream>>>(src, src_dtype, positions, table, table_dtype, table_rows, offset,
-                                                   out_f32, out_cd, cd_dtype, width);
+                                                   out_f32, out_cd, cd_dtype, width, scale);
   TNX_CHECK_LAUNCH("add_positions");
   return 0;
 }

@@ -1,0 +1,283 @@
+// A mixture of gated experts: the router's choice, the step's (token, choice) pairs put in the order of their
+// experts, and the two products of every expert over its own pairs,
+//     inner = act(w g) * (w u)  with [g | u] = W_gate_up[e] h      (the weight w on the expert's input; on its
+//     y = W_down[e] inner                                           output it multiplies y instead)
+// summed over a token's choices onto the residual in float32. Nothing is read back by the host: the launches are
+// sized by the most tiles the pairs can make, and a block that finds no tile ends at once.
+#include "common.h"
+
+TNX_DEFINE_ERROR_API
+
+#define TNX_ACT_SILU 4
+
+namespace {
+
+__device__ __forceinline__ float gate_act(float x, int act) {
+  if (act == TNX_ACT_SILU) return x / (1.f + expf(-x));
+  return apply_act(x, act);
+}
+
+// ---------------------------------------------------------------- the router's choice
+// A wave a token: scores sigmoid(z) or softmax(z), then `top` rounds of the largest score (the lower number where
+// two are equal).
+__global__ void __launch_bounds__(256) route_kernel(const float* __restrict__ z, int tokens, int experts, int top,
+                                                    int softmax, int renormalize, int* __restrict__ chosen,
+                                                    float* __restrict__ weights) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= tokens) return;
+  const float* row = z + (size_t)t * experts;
+  float peak = -INFINITY, total = 1.f;
+  if (softmax) {
+    for (int e = lane; e < experts; e += 64) peak = fmaxf(peak, row[e]);
+    peak = wave_max(peak);
+    float s = 0.f;
+    for (int e = lane; e < experts; e += 64) s += expf(row[e] - peak);
+    total = wave_sum(s);
+  }
+  auto score = [&](int e) { return softmax ? expf(row[e] - peak) / total : 1.f / (1.f + expf(-row[e])); };
+  float sum = 0.f;
+  unsigned long long taken = 0;        // bit i: expert lane + 64 i is chosen already (a lane's own experts)
+  for (int c = 0; c < top; ++c) {
+    float best = -1.f;
+    int at = experts;
+    for (int e = lane, i = 0; e < experts; e += 64, ++i) {
+      const float s = score(e);
+      if (!((taken >> i) & 1) && s > best) best = s, at = e;       // ascending e: the lower number stays where two are equal
+    }
+    const float high = wave_max(best);
+    const int first = -(int)wave_max((float)-(best == high ? at : experts));
+    if ((first & 63) == lane) taken |= 1ull << (first >> 6);
+    if (lane == 0) {
+      chosen[(size_t)t * top + c] = first;
+      weights[(size_t)t * top + c] = renormalize ? 0.f : high;
+    }
+    sum += high;
+  }
+  if (renormalize) {
+    // the same rounds again, now that the sum is known: each weight is written once
+    taken = 0;
+    for (int c = 0; c < top; ++c) {
+      float best = -1.f;
+      int at = experts;
+      for (int e = lane, i = 0; e < experts; e += 64, ++i) {
+        const float s = score(e);
+        if (!((taken >> i) & 1) && s > best) best = s, at = e;
+      }
+      const float high = wave_max(best);
+      const int first = -(int)wave_max((float)-(best == high ? at : experts));
+      if ((first & 63) == lane) taken |= 1ull << (first >> 6);
+      if (lane == 0) weights[(size_t)t * top + c] = high / sum;
+    }
+  }
+}
+
+// ---------------------------------------------------------------- pairs in the order of their experts
+// One block: counts an expert, where each expert's pairs begin (`first[E + 1]`), and the pairs (t * top + c)
+// put there (`order`). The order within an expert changes no result: every pair's row is computed alone.
+__global__ void __launch_bounds__(1024) order_kernel(const int* __restrict__ chosen, int pairs, int experts,
+                                                     int* __restrict__ first, int* __restrict__ order) {
+  extern __shared__ int counts[];      // [experts] counts, then [experts] cursors
+  int* cursor = counts + experts;
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    const int e = chosen[i];
+    if (e >= 0 && e < experts) atomicAdd(&counts[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < experts; ++e) {
+      first[e] = at;
+      cursor[e] = at;
+      at += counts[e];
+    }
+    first[experts] = at;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    const int e = chosen[i];
+    if (e >= 0 && e < experts) order[atomicAdd(&cursor[e], 1)] = i;
+  }
+}
+
+// ---------------------------------------------------------------- an expert's product over its pairs
+// out[pair, j] = sum_k A[row(pair), k] W[e][j][k] for the pairs of expert e, a tile of 16 pairs by 64 columns a
+// block, float32 sums from tiles staged in LDS. GATED: W holds F gate rows and then F up rows, column j of the
+// result is act(w g_j) * (w u_j) and the A row of a pair is its token's (pair / top). Otherwise the A row is the
+// pair's own, and the result goes to `out` (pair rows, float32) or, where a token has one choice, straight onto
+// the residual into the token's row.
+struct ProductArgs {
+  const void* a;            // GATED: h [T, K]; else inner [pairs, K]
+  const void* w;            // [E, N(, 2), K]
+  const int* first;         // [E + 1]
+  const int* order;         // [pairs]
+  const float* weights;     // [pairs]
+  const float* residual;    // [T, N] or null (not GATED, one choice a token)
+  void* out;
+  int experts, top, n, k, act, weight_on_input, pairs;
+};
+
+template <typename T, bool GATED>
+__global__ void __launch_bounds__(256) expert_product_kernel(ProductArgs p) {
+  constexpr int TM = 16, TN = 64, TK = 32;
+  __shared__ float As[TM][TK + 1];
+  __shared__ float Ws[GATED ? 2 : 1][TN][TK + 1];
+  __shared__ int rows[TM];
+  // which expert and which of its tiles of 16 pairs this block is
+  int tile = blockIdx.y, e = 0, begin = 0, end = 0;
+  for (; e < p.experts; ++e) {
+    begin = p.first[e];
+    end = p.first[e + 1];
+    const int tiles = (end - begin + TM - 1) / TM;
+    if (tile < tiles) break;
+    tile -= tiles;
+  }
+  if (e >= p.experts) return;
+  begin += tile * TM;
+  const int count = min(TM, end - begin);
+  const int col0 = blockIdx.x * TN;
+  if (threadIdx.x < TM) rows[threadIdx.x] = threadIdx.x < count ? p.order[begin + threadIdx.x] : -1;
+  __syncthreads();
+  const T* A = (const T*)p.a;
+  const T* W = (const T*)p.w + (size_t)e * (GATED ? 2 : 1) * p.n * p.k;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;        // column, and rows 4 ty .. 4 ty + 3
+  float acc[GATED ? 2 : 1][4] = {};
+  for (int k0 = 0; k0 < p.k; k0 += TK) {
+    // the tile of A: 16 rows of 32, two elements a thread
+    for (int i = threadIdx.x; i < TM * TK; i += 256) {
+      const int r = i / TK, c = i - r * TK;
+      const int pair = rows[r];
+      float v = 0.f;
+      if (pair >= 0 && k0 + c < p.k) v = to_f32(A[(size_t)(GATED ? pair / p.top : pair) * p.k + k0 + c]);
+      As[r][c] = v;
+    }
+    // the tile of W: 64 (or twice 64) rows of 32
+    for (int i = threadIdx.x; i < (GATED ? 2 : 1) * TN * TK; i += 256) {
+      const int half = i / (TN * TK), j = (i - half * TN * TK) / TK, c = i % TK;
+      float v = 0.f;
+      if (col0 + j < p.n && k0 + c < p.k) v = to_f32(W[((size_t)half * p.n + col0 + j) * p.k + k0 + c]);
+      Ws[half][j][c] = v;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int c = 0; c < TK; ++c) {
+      const float w0 = Ws[0][tx][c];
+      const float w1 = GATED ? Ws[GATED ? 1 : 0][tx][c] : 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float x = As[4 * ty + r][c];
+        acc[0][r] += x * w0;
+        if (GATED) acc[GATED ? 1 : 0][r] += x * w1;
+      }
+    }
+    __syncthreads();
+  }
+  const int col = col0 + tx;
+  if (col >= p.n) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int pair = rows[4 * ty + r];
+    if (pair < 0) continue;
+    const float w = p.weights[pair];
+    if (GATED) {
+      float g = acc[0][r], u = acc[GATED ? 1 : 0][r];
+      if (p.weight_on_input) g *= w, u *= w;
+      ((T*)p.out)[(size_t)pair * p.n + col] = from_f32<T>(gate_act(g, p.act) * u);
+    } else {
+      float y = acc[0][r];
+      if (!p.weight_on_input) y *= w;
+      if (p.top == 1)
+        ((float*)p.out)[(size_t)pair * p.n + col] = y + (p.residual ? p.residual[(size_t)pair * p.n + col] : 0.f);
+      else
+        ((float*)p.out)[(size_t)pair * p.n + col] = y;
+    }
+  }
+}
+
+// out[t] = residual[t] + sum_c y[t * top + c], in the order of c
+__global__ void combine_kernel(const float* __restrict__ y, const float* __restrict__ residual, float* __restrict__ out,
+                               int top, size_t n, size_t total) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += stride) {
+    const size_t t = i / n, col = i - t * n;
+    float s = residual ? residual[i] : 0.f;
+    for (int c = 0; c < top; ++c) s += y[(t * top + c) * n + col];
+    out[i] = s;
+  }
+}
+
+// act(g) * u from rows [g | u] of float32
+template <typename T>
+__global__ void gated_activation_kernel(const float* __restrict__ gu, T* __restrict__ out, int f, int act, size_t total) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += stride) {
+    const size_t t = i / f, j = i - t * f;
+    out[i] = from_f32<T>(gate_act(gu[t * 2 * f + j], act) * gu[t * 2 * f + f + j]);
+  }
+}
+
+int blocks_for(size_t total) {
+  size_t b = (total + 255) / 256;
+  return (int)(b > 16384 ? 16384 : (b ? b : 1));
+}
+
+}  // namespace
+
+extern "C" int tnx_route(const float* z, int tokens, int experts, int top, int softmax, int renormalize, int* chosen,
+                         float* weights, hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && experts > 0 && top > 0 && top <= experts, "route: %d of %d experts", top, experts);
+  if (tokens == 0) return 0;
+  route_kernel<<<(tokens + 3) / 4, 256, 0, stream>>>(z, tokens, experts, top, softmax, renormalize, chosen, weights);
+  TNX_CHECK_LAUNCH("route");
+  return 0;
+}
+
+extern "C" int tnx_expert_mixture(const void* h, const int* chosen, const float* weights, const void* w_gate_up,
+                                  const void* w_down, int* first, int* order, void* inner, float* pair_rows,
+                                  const float* residual, float* out, int dtype, int tokens, int experts, int top,
+                                  int width, int f, int act, int weight_on_input, hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && experts > 0 && top > 0 && width > 0 && f > 0, "expert_mixture: bad sizes");
+  TNX_REQUIRE(experts <= 4096, "expert_mixture: up to 4096 experts, got %d", experts);
+  TNX_REQUIRE(dtype == TNX_F32 || dtype == TNX_BF16, "expert_mixture: dtype %d", dtype);
+  TNX_REQUIRE(top == 1 || pair_rows != nullptr, "expert_mixture: several choices a token need room for their rows");
+  if (tokens == 0) return 0;
+  const int pairs = tokens * top;
+  order_kernel<<<1, 1024, 2 * experts * sizeof(int), stream>>>(chosen, pairs, experts, first, order);
+  TNX_CHECK_LAUNCH("expert order");
+  const int tiles = pairs / 16 + experts;       // the most tiles of 16 pairs: every expert may end in a part of one
+  ProductArgs up{h, w_gate_up, first, order, weights, nullptr, inner, experts, top, f, width, act, weight_on_input, pairs};
+  ProductArgs down{inner, w_down, first, order, weights, residual, top == 1 ? out : pair_rows, experts, top, width, f,
+                   act, weight_on_input, pairs};
+  const dim3 grid_up((f + 63) / 64, tiles), grid_down((width + 63) / 64, tiles);
+  if (dtype == TNX_F32) {
+    expert_product_kernel<float, true><<<grid_up, 256, 0, stream>>>(up);
+    expert_product_kernel<float, false><<<grid_down, 256, 0, stream>>>(down);
+  } else {
+    expert_product_kernel<bf16_t, true><<<grid_up, 256, 0, stream>>>(up);
+    expert_product_kernel<bf16_t, false><<<grid_down, 256, 0, stream>>>(down);
+  }
+  TNX_CHECK_LAUNCH("expert products");
+  if (top > 1) {
+    const size_t total = (size_t)tokens * width;
+    combine_kernel<<<blocks_for(total), 256, 0, stream>>>(pair_rows, residual, out, top, (size_t)width, total);
+    TNX_CHECK_LAUNCH("expert combine");
+  }
+  return 0;
+}
+
+extern "C" int tnx_gated_activation(const float* gate_up, void* out, int dtype, int tokens, int f, int act,
+                                    hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && f > 0, "gated_activation: bad sizes");
+  TNX_REQUIRE(dtype == TNX_F32 || dtype == TNX_BF16, "gated_activation: dtype %d", dtype);
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * f;
+  if (dtype == TNX_F32)
+    gated_activation_kernel<float><<<blocks_for(total), 256, 0, stream>>>(gate_up, (float*)out, f, act, total);
+  else
+    gated_activation_kernel<bf16_t><<<blocks_for(total), 256, 0, stream>>>(gate_up, (bf16_t*)out, f, act, total);
+  TNX_CHECK_LAUNCH("gated_activation");
+  return 0;
+}

@@ -17,6 +17,7 @@ from .. import debug
 
 _F32, _BF16 = 0, 1
 _ACT = {None: 0, "none": 0, "relu": 1, "gelu": 2, "gelu_new": 3}
+_GATE_ACT = {"gelu_new": 3, "silu": 4}     # what a gated expert's kernels take
 _LIBS: Dict[str, ctypes.CDLL] = {}
 
 _c_void_p, _c_int, _c_float, _c_ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_longlong
@@ -27,7 +28,7 @@ _SIGNATURES = {
         "tnx_copy_ints": [_c_void_p, _c_void_p, _c_int, _c_void_p],
         "tnx_device_pointer": [_c_void_p, _c_void_p],
         "tnx_add_positions": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
-                              _c_int, _c_int, _c_int, _c_void_p],
+                              _c_int, _c_int, _c_int, _c_float, _c_void_p],
         "tnx_cast": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_void_p],
         "tnx_epilogue": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_layernorm": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
@@ -114,6 +115,23 @@ _SIGNATURES = {
         "tnx_latent_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                                      _c_int, _c_int, _c_void_p, _c_void_p, _c_ll, _c_ll, _c_void_p, _c_int, _c_float,
                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    },
+    "prepare": {
+        "tnx_qkv_prepare": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_void_p,
+                            _c_float, _c_void_p, _c_void_p, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                            _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    },
+    "memory": {
+        "tnx_matrix_memory": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                              _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                              _c_int, _c_float, _c_void_p],
+    },
+    "experts": {
+        "tnx_route": [_c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
+        "tnx_expert_mixture": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                               _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                               _c_int, _c_void_p],
+        "tnx_gated_activation": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "probe": {
         "tnx_probe_stream_read": [_c_void_p, ctypes.c_size_t, _c_void_p, _c_int, _c_void_p],
@@ -394,7 +412,7 @@ class HipOps:
         self._call("sampling", "tnx_store_tokens", _ptr(tokens), _ptr(ctx.logits_rows), _ptr(ctx.token_request),
                    _ptr(ctx.slots), tokens.numel(), _ptr(kept), kept.numel(), landing, _stream())
 
-    def add_positions(self, src, positions, table, offset, dtype, want_compute):
+    def add_positions(self, src, positions, table, offset, dtype, want_compute, scale=1.0):
         _want(src, "src")
         t, width = src.shape
         _want(positions, "positions", torch.int32, (t,))
@@ -404,16 +422,17 @@ class HipOps:
         out = torch.empty(t, width, dtype=torch.float32, device=src.device)
         cd = torch.empty(t, width, dtype=dtype, device=src.device) if want_compute and dtype != torch.float32 else None
         self._call("elementwise", "tnx_add_positions", _ptr(src), _code(src.dtype), _ptr(positions), _ptr(table),
-                   _code(table.dtype), table.shape[0], offset, _ptr(out), _ptr(cd), _code(dtype), t, width, _stream())
+                   _code(table.dtype), table.shape[0], offset, _ptr(out), _ptr(cd), _code(dtype), t, width, float(scale),
+                   _stream())
         return out, ((cd if cd is not None else out) if want_compute else None)
 
-    def to_stream(self, src, dtype, want_compute):
+    def to_stream(self, src, dtype, want_compute, scale=1.0):
         _want(src, "src")
         t, width = src.shape
         out = torch.empty(t, width, dtype=torch.float32, device=src.device)
         cd = torch.empty(t, width, dtype=dtype, device=src.device) if want_compute and dtype != torch.float32 else None
         self._call("elementwise", "tnx_add_positions", _ptr(src), _code(src.dtype), None, None, 0, 0, 0, _ptr(out),
-                   _ptr(cd), _code(dtype), t, width, _stream())
+                   _ptr(cd), _code(dtype), t, width, float(scale), _stream())
         return out, ((cd if cd is not None else out) if want_compute else None)
 
     def cast(self, x, dtype):
@@ -1348,6 +1367,117 @@ class HipOps:
                    num_pages, _ptr(latent_pages), _ptr(rotated_pages), latent_pages.stride(0), rotated_pages.stride(0),
                    _ptr(freqs), freqs.numel(), float(scale), num_heads, head_size, rot, kv_rank, int(window or 0), t,
                    _stream())
+        return out
+
+
+    # ---------------------------------------------------------------- normed, turned and blended projections
+
+    def qkv_prepare(self, proj, num_heads, num_kv, head_size, value_size, cache_head, q_weight, k_weight, eps, freqs,
+                    interleaved, scale, mix_weight, first_values, ctx, view, k_pages, v_pages):
+        """See `ReferenceOps.qkv_prepare`."""
+        t = ctx.num_tokens
+        total = num_heads * head_size + num_kv * (head_size + value_size)
+        _want(proj, "projections", torch.float32, (t, total))
+        if q_weight is not None:
+            _want(q_weight, "query norm", torch.float32, (num_heads * head_size,))
+            _want(k_weight, "key norm", torch.float32, (num_kv * head_size,))
+        if freqs is not None:
+            _want(freqs, "frequencies", torch.float32)
+        first_ld = 0
+        if first_values is not None:
+            _want(mix_weight, "blending weight", torch.float32, (1,))
+            if (not first_values.is_cuda or first_values.dtype != torch.float32 or first_values.dim() != 2
+                    or tuple(first_values.shape) != (t, num_kv * value_size) or first_values.stride(1) != 1):
+                raise ValueError(f"the values to blend with are float32 [{t}, {num_kv * value_size}] with dense rows, got "
+                                 f"{tuple(first_values.shape)} {first_values.dtype}")
+            first_ld = first_values.stride(0)
+        num_pages = self._check_pages(k_pages, v_pages, num_kv, cache_head, view.page_size)
+        _want(view.token_page, "token pages", torch.int32, (t,))
+        _want(view.token_offset, "token offsets", torch.int32, (t,))
+        q = torch.empty(t, num_heads * cache_head, dtype=self.dtype, device=proj.device)
+        self._call("prepare", "tnx_qkv_prepare", _ptr(proj), total, _ptr(q_weight), _ptr(k_weight), float(eps),
+                   _ptr(freqs), freqs.numel() if freqs is not None else 0, int(bool(interleaved)), _ptr(ctx.positions),
+                   float(scale), _ptr(mix_weight) if first_values is not None else None, _ptr(first_values), first_ld,
+                   _ptr(view.token_page), _ptr(view.token_offset), _ptr(q), _ptr(k_pages), _ptr(v_pages),
+                   k_pages.stride(0), num_pages, view.page_size, _code(self.dtype), t, num_heads, num_kv, head_size,
+                   value_size, cache_head, _stream(),
+                   work=(f"{t}x{total}", t * (total * 4 + (num_heads + 2 * num_kv) * cache_head * q.element_size()), 0.0))
+        return q
+
+    # ---------------------------------------------------------------- the matrix memory
+
+    def matrix_memory(self, proj, num_heads, head_size, value_size, gate_cap, eps, norm_weight, ctx, memory, normalizer,
+                      peak):
+        """See `ReferenceOps.matrix_memory`."""
+        t = ctx.num_tokens
+        h, n, v = num_heads, head_size, value_size
+        total = 2 * h * n + 2 * h * v + 2 * h
+        _want(proj, "projections", torch.float32, (t, total))
+        _want(norm_weight, "norm weight", torch.float32, (h * v,))
+        slots = memory.shape[0]
+        _want(memory, "memory", torch.float32, (slots, 2, h, n, v))
+        _want(normalizer, "normalizer", torch.float32, (slots, 2, h, n))
+        _want(peak, "peak", torch.float32, (slots, 2, h))
+        raw = torch.empty(t, h * v, dtype=torch.float32, device=proj.device)
+        out = torch.empty(t, h * v, dtype=self.dtype, device=proj.device)
+        state = float(ctx.num_requests) * h * n * v * 8
+        self._call("memory", "tnx_matrix_memory", _ptr(proj), total, _ptr(ctx.run_start), _ptr(ctx.cached_lens),
+                   _ptr(ctx.slots), _ptr(memory), _ptr(normalizer), _ptr(peak), slots, _ptr(raw), _ptr(norm_weight),
+                   float(eps), _ptr(out), _code(self.dtype), t, ctx.num_requests, h, n, v, float(gate_cap), _stream(),
+                   work=(f"{t} tokens {ctx.num_requests} runs", state + t * total * 4.0, 4.0 * t * h * n * v))
+        return out
+
+    # ---------------------------------------------------------------- experts
+
+    def route(self, z, top, score="sigmoid", renormalize=False):
+        """See `ReferenceOps.route`."""
+        _want(z, "router logits", torch.float32)
+        t, experts = z.shape
+        if score not in ("sigmoid", "softmax"):
+            raise ValueError(f"unknown router score {score!r}")
+        chosen = torch.empty(t, top, dtype=torch.int32, device=z.device)
+        weights = torch.empty(t, top, dtype=torch.float32, device=z.device)
+        self._call("experts", "tnx_route", _ptr(z), t, experts, top, int(score == "softmax"), int(bool(renormalize)),
+                   _ptr(chosen), _ptr(weights), _stream())
+        return chosen, weights
+
+    def gated_activation(self, gate_up, activation):
+        """See `ReferenceOps.gated_activation`."""
+        _want(gate_up, "gate and up", torch.float32)
+        t, two_f = gate_up.shape
+        if two_f % 2 or activation not in _GATE_ACT:
+            raise ValueError(f"gated_activation: rows of {two_f}, activation {activation!r}")
+        out = torch.empty(t, two_f // 2, dtype=self.dtype, device=gate_up.device)
+        self._call("experts", "tnx_gated_activation", _ptr(gate_up), _ptr(out), _code(self.dtype), t, two_f // 2,
+                   _GATE_ACT[activation], _stream(), work=(f"{t}x{two_f // 2}", t * two_f * 4.0 + out.numel() * out.element_size(), 0.0))
+        return out
+
+    def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None):
+        """See `ReferenceOps.expert_mixture`."""
+        t, top = chosen.shape
+        experts, two_f, width = w_gate_up.shape
+        f = two_f // 2
+        if activation not in _GATE_ACT or weight_on not in ("input", "output"):
+            raise ValueError(f"expert_mixture: activation {activation!r}, weight_on {weight_on!r}")
+        _want(h, "h", w_gate_up.dtype, (t, width))
+        _want(chosen, "chosen experts", torch.int32)
+        _want(weights, "weights", torch.float32, (t, top))
+        _want(w_gate_up, "gate and up matrices")
+        _want(w_down, "down matrices", w_gate_up.dtype, (experts, width, f))
+        if residual is not None:
+            _want(residual, "residual", torch.float32, (t, width))
+        dev = h.device
+        ints = torch.empty(experts + 1 + t * top, dtype=torch.int32, device=dev)
+        inner = torch.empty(t * top, f, dtype=h.dtype, device=dev)
+        rows = torch.empty(t * top, width, dtype=torch.float32, device=dev) if top > 1 else None
+        out = torch.empty(t, width, dtype=torch.float32, device=dev)
+        item = h.element_size()
+        used = min(experts, t * top)
+        self._call("experts", "tnx_expert_mixture", _ptr(h), _ptr(chosen), _ptr(weights), _ptr(w_gate_up), _ptr(w_down),
+                   _ptr(ints[:experts + 1]), _ptr(ints[experts + 1:]), _ptr(inner), _ptr(rows), _ptr(residual), _ptr(out),
+                   _code(h.dtype), t, experts, top, width, f, _GATE_ACT[activation], int(weight_on == "input"), _stream(),
+                   work=(f"{t}x{top} of {experts}", used * 3.0 * f * width * item + t * width * (item + 8.0),
+                         6.0 * t * top * f * width))
         return out
 
     # ---------------------------------------------------------------- output end
