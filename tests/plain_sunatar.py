@@ -186,7 +186,7 @@ def mixture(mlp, w, p, h):
 def forward(cfg, w, tokens, return_layers=False):
     """Logits `[T, vocab]` of a whole sequence; with `return_layers` also the stream after every layer."""
     eps = cfg["norm"]["eps"]
-    x = w["embed"][torch.tensor(tokens)] * cfg["embedding"]["scale"]
+    x = w["embed"][torch.tensor(tokens)] * (cfg.get("embedding") or {}).get("scale", 1.0)
     v_first = None
     streams = []
     for i, layer in enumerate(cfg["layers"]):

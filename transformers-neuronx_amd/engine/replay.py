@@ -29,7 +29,8 @@ from .factory import runner_from_folder
 def make_replay_runner(model_dir: str, dtype: str, max_tokens: int, page_size: int = 64, device: str = "cuda:0",
                        kernels: str = "hip", max_requests: int = 16):
     """The runner a replay uses: a page pool for `max_tokens` tokens (each
-    request's count rounded up to whole pages by the caller)."""
+    request's count rounded up to whole pages by the caller) and state slots for
+    `max_requests` requests, so that pages and slots change hands during a trace."""
     cfg = EngineConfig(dtype=dtype, page_size=page_size, max_tokens=max_tokens, max_num_seqs=max_requests,
                        device=device, kernels=kernels)
     return runner_from_folder(model_dir, cfg)
@@ -71,6 +72,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="the most tokens live requests hold at a time (each request's count in whole pages)")
     ap.add_argument("--page-size", type=int, default=64, help="tokens per cache page (divides 64 or is a multiple)")
+    ap.add_argument("--max-requests", type=int, default=4, help="the most requests that are live at a time")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
     if not os.environ.get("HOME") or not os.access(os.environ.get("HOME", "/"), os.W_OK):
@@ -78,7 +80,8 @@ def main(argv=None) -> int:
         import tempfile
         os.environ["HOME"] = tempfile.mkdtemp(prefix="trace_run_home_")
     print("[trace_run] loading the model ...", file=sys.stderr, flush=True)
-    runner = make_replay_runner(args.model, args.dtype, args.max_tokens, args.page_size, args.device)
+    runner = make_replay_runner(args.model, args.dtype, args.max_tokens, args.page_size, args.device,
+                                max_requests=args.max_requests)
     print("[trace_run] ready", file=sys.stderr, flush=True)
     replay(sys.stdin, runner, args.out)
     return 0

@@ -170,6 +170,8 @@ class ReferenceOps:
             pages = view.block_table[r, :nb].long().clamp(min=0)
             keys = k_pages[pages].float().permute(1, 0, 2, 3).reshape(num_kv_heads, nb * ps, head_size)[:, :total]
             vals = v_pages[pages].float().permute(1, 2, 0, 3).reshape(num_kv_heads, head_size, nb * ps)[:, :, :total]
+            # pages that were given back may hold anything: what the mask hides must not reach the sum
+            vals = torch.where(torch.isfinite(vals), vals, torch.zeros_like(vals))
             qr = q[s:e].float().reshape(e - s, num_heads, head_size).permute(1, 0, 2)
             keys = keys.repeat_interleave(group, dim=0)
             vals = vals.repeat_interleave(group, dim=0)

@@ -106,12 +106,13 @@ class SunatarConfig(ModelConfig):
                 if "v_mix" in m and not isinstance(m["v_mix"], bool):
                     raise ConfigError(f"key '{where}.mixer.v_mix' must be true or false, got {m['v_mix']!r}")
                 if m.get("v_mix"):
-                    mine = groups * m["vdim"]
+                    mine = (groups, m["vdim"])
                     if mixed is None:
                         mixed = (i, mine)
                     elif mixed[1] != mine:
-                        raise ConfigError(f"key '{where}.mixer': its values ({mine} a token) are blended with those of "
-                                          f"layer {mixed[0]} ({mixed[1]} a token); kv_heads * vdim must agree")
+                        raise ConfigError(f"key '{where}.mixer': its values ({mine[0]} heads of {mine[1]}) are blended with "
+                                          f"those of layer {mixed[0]} ({mixed[1][0]} heads of {mixed[1][1]}); kv_heads and "
+                                          f"vdim must agree")
             else:
                 _need(m, "gate_cap", float, where + ".mixer")
             mlp = layer.get("mlp")
