@@ -61,10 +61,29 @@ def ratesun_config(width, heads, ff, vocab, layers, q_rank, window=1024):
                              mlp=dict(kind="dense", ff=ff)) for i in range(layers)])
 
 
+def sunatar_config(width, heads, head, ff, vocab, layers, window=1024):
+    """config.json contents of a Sunatar model at the sizes of a published layer: every fourth layer (the second
+    first) a matrix memory of `heads` heads of 64 by `head`, the others attention over a window with a quarter as
+    many key/value heads as query heads; every layer's feed-forward eight experts of ff / 4 of which a token takes
+    two, beside a shared one of ff / 2: a token meets an inner size of `ff`, as the other design's does."""
+    attention = dict(heads=heads, kv_heads=max(1, heads // 4), dim=head, vdim=head, scale=head ** -0.5, v_mix=True,
+                     mask=dict(size=window), rot=dict(base=10000.0, dims=head // 2,
+                                                      scaling=dict(factor=4.0, low=1.0, high=4.0, original=2048)))
+    memory = dict(heads=heads, dim=64, vdim=head, gate_cap=15.0)
+    mlp = dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=ff // 4), shared=dict(ff=ff // 2))
+    return dict(architecture="Sunatar", vocab=vocab, width=width, norm=dict(eps=1e-5), embedding=dict(scale=1.0),
+                init_std=0.02, max_positions=4096,
+                layers=[dict(type="mlstm", mixer=memory, mlp=mlp) if i % 4 == 1 else
+                        dict(type="attention", mixer=attention, mlp=mlp) for i in range(layers)])
+
+
 # a new design beside the closest one the engine had, at equal sizes: {design: {size: (its config, the other's)}}
 BESIDE = {"ratesun": {
     "2048 wide": (lambda n: ratesun_config(2048, 16, 8192, 50272, n, 768), "1.3b"),
     "4096 wide": (lambda n: ratesun_config(4096, 32, 16384, 50272, n, 1536), "6.7b"),
+}, "sunatar": {
+    "2048 wide": (lambda n: sunatar_config(2048, 32, 64, 8192, 50272, n), "1.3b"),
+    "4096 wide": (lambda n: sunatar_config(4096, 32, 128, 16384, 50272, n), "6.7b"),
 }}
 PREFILL_TOKENS = 2048
 PEAK_HBM_GBS = 8000.0                      # MI355X, published

@@ -75,7 +75,9 @@ __global__ void __launch_bounds__(256) route_kernel(const float* __restrict__ z,
 // One block: counts an expert, where each expert's pairs begin (`first[E + 1]`), and the pairs (t * top + c)
 // put there (`order`). The order within an expert changes no result: every pair's row is computed alone.
 __global__ void __launch_bounds__(1024) order_kernel(const int* __restrict__ chosen, int pairs, int experts,
-                                                     int* __restrict__ first, int* __restrict__ order) {
+                                                     int* __restrict__ first, int* __restrict__ order,
+                                                     int* __restrict__ place, int* __restrict__ token, int top,
+                                                     const float* __restrict__ weights, float* __restrict__ sorted_weights) {
   extern __shared__ int counts[];      // [experts] counts, then [experts] cursors
   int* cursor = counts + experts;
   for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
@@ -97,7 +99,13 @@ __global__ void __launch_bounds__(1024) order_kernel(const int* __restrict__ cho
   __syncthreads();
   for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
     const int e = chosen[i];
-    if (e >= 0 && e < experts) order[atomicAdd(&cursor[e], 1)] = i;
+    if (e >= 0 && e < experts) {
+      const int at = atomicAdd(&cursor[e], 1);
+      order[at] = i;
+      if (place) place[i] = at;                       // where the pair's row lies among the sorted ones
+      if (token) token[at] = i / top;                 // the token whose row the sorted row reads
+      if (sorted_weights) sorted_weights[at] = weights[i];
+    }
   }
 }
 
@@ -195,27 +203,98 @@ __global__ void __launch_bounds__(256) expert_product_kernel(ProductArgs p) {
   }
 }
 
+
+// The same tile on the matrix unit, bfloat16 with an inner size in 8s: a wave takes 16 columns (and with GATED the
+// 16 up rows that go with its 16 gate rows) for the tile's 16 pairs and makes out^T[column][pair] with MFMA
+// 16x16x32, the matrix's rows as the A operand, 16 bytes a lane as they lie and read once, the pairs' rows as the B
+// operand. Nothing goes through LDS: an expert's matrix is read once for every 16 of its pairs, which in a decode
+// step is once, and the rows of the pairs come from the caches.
+template <bool GATED>
+__global__ void __launch_bounds__(256) expert_product_mfma_kernel(ProductArgs p) {
+  constexpr int TM = 16;
+  int tile = blockIdx.y, e = 0, begin = 0, end = 0;
+  for (; e < p.experts; ++e) {
+    begin = p.first[e];
+    end = p.first[e + 1];
+    const int tiles = (end - begin + TM - 1) / TM;
+    if (tile < tiles) break;
+    tile -= tiles;
+  }
+  if (e >= p.experts) return;
+  begin += tile * TM;
+  const int count = min(TM, end - begin);
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int col0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 16;
+  if (col0 >= p.n) return;
+  const int pair = r < count ? p.order[begin + r] : -1;
+  const bf16_t* xrow = (const bf16_t*)p.a + (size_t)(pair < 0 ? 0 : (GATED ? pair / p.top : pair)) * p.k;
+  const bf16_t* W = (const bf16_t*)p.w + (size_t)e * (GATED ? 2 : 1) * p.n * p.k;
+  const int n = col0 + r;
+  const bf16_t* wrow = W + (size_t)min(n, p.n - 1) * p.k;
+  const bf16_t* urow = wrow + (size_t)p.n * p.k;          // GATED: the up row of the same column
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc_up = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int k0 = 0; k0 < p.k; k0 += 32) {
+    const int d0 = k0 + 8 * g;
+    const bool in = d0 < p.k;
+    const bf16x8 b = (in && pair >= 0) ? *(const bf16x8*)(xrow + d0) : zero8;
+    const bf16x8 a = (in && n < p.n) ? load_once(wrow + d0) : zero8;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+    if (GATED) {
+      const bf16x8 u = (in && n < p.n) ? load_once(urow + d0) : zero8;
+      acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u, b, acc_up, 0, 0, 0);
+    }
+  }
+  if (pair < 0) return;
+  const float w = p.weights[pair];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int col = col0 + 4 * g + i;        // the lane holds columns 4 g .. 4 g + 3 of pair r
+    if (col >= p.n) continue;
+    if (GATED) {
+      float gt = acc[i], up = acc_up[i];
+      if (p.weight_on_input) gt *= w, up *= w;
+      ((bf16_t*)p.out)[(size_t)pair * p.n + col] = (bf16_t)(gate_act(gt, p.act) * up);
+    } else {
+      float y = acc[i];
+      if (!p.weight_on_input) y *= w;
+      if (p.top == 1 && p.residual) y += p.residual[(size_t)pair * p.n + col];
+      ((float*)p.out)[(size_t)pair * p.n + col] = y;
+    }
+  }
+}
+
 // out[t] = residual[t] + sum_c y[t * top + c], in the order of c
+// (`place`: the row of y that holds pair t * top + c, where the rows lie in another order; `scale`: a factor a pair)
 __global__ void combine_kernel(const float* __restrict__ y, const float* __restrict__ residual, float* __restrict__ out,
-                               int top, size_t n, size_t total) {
+                               int top, size_t n, size_t total, const int* __restrict__ place,
+                               const float* __restrict__ scale) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (; i < total; i += stride) {
     const size_t t = i / n, col = i - t * n;
     float s = residual ? residual[i] : 0.f;
-    for (int c = 0; c < top; ++c) s += y[(t * top + c) * n + col];
+    for (int c = 0; c < top; ++c) {
+      const size_t pair = t * top + c;
+      const float v = y[(place ? (size_t)place[pair] : pair) * n + col];
+      s += scale ? scale[pair] * v : v;
+    }
     out[i] = s;
   }
 }
 
 // act(g) * u from rows [g | u] of float32
+// (`row_weights`: a factor a row on both g and u, the weight on an expert's input)
 template <typename T>
-__global__ void gated_activation_kernel(const float* __restrict__ gu, T* __restrict__ out, int f, int act, size_t total) {
+__global__ void gated_activation_kernel(const float* __restrict__ gu, T* __restrict__ out, int f, int act, size_t total,
+                                        const float* __restrict__ row_weights) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (; i < total; i += stride) {
     const size_t t = i / f, j = i - t * f;
-    out[i] = from_f32<T>(gate_act(gu[t * 2 * f + j], act) * gu[t * 2 * f + f + j]);
+    const float w = row_weights ? row_weights[t] : 1.f;
+    out[i] = from_f32<T>(gate_act(w * gu[t * 2 * f + j], act) * (w * gu[t * 2 * f + f + j]));
   }
 }
 
@@ -238,14 +317,15 @@ extern "C" int tnx_route(const float* z, int tokens, int experts, int top, int s
 extern "C" int tnx_expert_mixture(const void* h, const int* chosen, const float* weights, const void* w_gate_up,
                                   const void* w_down, int* first, int* order, void* inner, float* pair_rows,
                                   const float* residual, float* out, int dtype, int tokens, int experts, int top,
-                                  int width, int f, int act, int weight_on_input, hipStream_t stream) {
+                                  int width, int f, int act, int weight_on_input, int plain, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && experts > 0 && top > 0 && width > 0 && f > 0, "expert_mixture: bad sizes");
   TNX_REQUIRE(experts <= 4096, "expert_mixture: up to 4096 experts, got %d", experts);
   TNX_REQUIRE(dtype == TNX_F32 || dtype == TNX_BF16, "expert_mixture: dtype %d", dtype);
   TNX_REQUIRE(top == 1 || pair_rows != nullptr, "expert_mixture: several choices a token need room for their rows");
   if (tokens == 0) return 0;
   const int pairs = tokens * top;
-  order_kernel<<<1, 1024, 2 * experts * sizeof(int), stream>>>(chosen, pairs, experts, first, order);
+  order_kernel<<<1, 1024, 2 * experts * sizeof(int), stream>>>(chosen, pairs, experts, first, order, nullptr, nullptr,
+                                                               top, nullptr, nullptr);
   TNX_CHECK_LAUNCH("expert order");
   const int tiles = pairs / 16 + experts;       // the most tiles of 16 pairs: every expert may end in a part of one
   ProductArgs up{h, w_gate_up, first, order, weights, nullptr, inner, experts, top, f, width, act, weight_on_input, pairs};
@@ -255,6 +335,9 @@ extern "C" int tnx_expert_mixture(const void* h, const int* chosen, const float*
   if (dtype == TNX_F32) {
     expert_product_kernel<float, true><<<grid_up, 256, 0, stream>>>(up);
     expert_product_kernel<float, false><<<grid_down, 256, 0, stream>>>(down);
+  } else if (width % 8 == 0 && f % 8 == 0 && !plain) {
+    expert_product_mfma_kernel<true><<<grid_up, 256, 0, stream>>>(up);
+    expert_product_mfma_kernel<false><<<grid_down, 256, 0, stream>>>(down);
   } else {
     expert_product_kernel<bf16_t, true><<<grid_up, 256, 0, stream>>>(up);
     expert_product_kernel<bf16_t, false><<<grid_down, 256, 0, stream>>>(down);
@@ -262,22 +345,48 @@ extern "C" int tnx_expert_mixture(const void* h, const int* chosen, const float*
   TNX_CHECK_LAUNCH("expert products");
   if (top > 1) {
     const size_t total = (size_t)tokens * width;
-    combine_kernel<<<blocks_for(total), 256, 0, stream>>>(pair_rows, residual, out, top, (size_t)width, total);
+    combine_kernel<<<blocks_for(total), 256, 0, stream>>>(pair_rows, residual, out, top, (size_t)width, total, nullptr,
+                                                          nullptr);
     TNX_CHECK_LAUNCH("expert combine");
   }
   return 0;
 }
 
 extern "C" int tnx_gated_activation(const float* gate_up, void* out, int dtype, int tokens, int f, int act,
-                                    hipStream_t stream) {
+                                    const float* row_weights, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && f > 0, "gated_activation: bad sizes");
   TNX_REQUIRE(dtype == TNX_F32 || dtype == TNX_BF16, "gated_activation: dtype %d", dtype);
   if (tokens == 0) return 0;
   const size_t total = (size_t)tokens * f;
   if (dtype == TNX_F32)
-    gated_activation_kernel<float><<<blocks_for(total), 256, 0, stream>>>(gate_up, (float*)out, f, act, total);
+    gated_activation_kernel<float><<<blocks_for(total), 256, 0, stream>>>(gate_up, (float*)out, f, act, total, row_weights);
   else
-    gated_activation_kernel<bf16_t><<<blocks_for(total), 256, 0, stream>>>(gate_up, (bf16_t*)out, f, act, total);
+    gated_activation_kernel<bf16_t><<<blocks_for(total), 256, 0, stream>>>(gate_up, (bf16_t*)out, f, act, total,
+                                                                            row_weights);
   TNX_CHECK_LAUNCH("gated_activation");
+  return 0;
+}
+
+// The pairs in the order of their experts, for a caller that runs the experts' products itself: `first[E + 1]`,
+// `order[pairs]`, `place[pairs]` (where a pair went), `token[pairs]` (the token of each sorted row) and the weights in
+// sorted order.
+extern "C" int tnx_expert_order(const int* chosen, const float* weights, int tokens, int experts, int top, int* first,
+                                int* order, int* place, int* token, float* sorted_weights, hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && experts > 0 && experts <= 4096 && top > 0, "expert_order: bad sizes");
+  if (tokens == 0) return 0;
+  order_kernel<<<1, 1024, 2 * experts * sizeof(int), stream>>>(chosen, tokens * top, experts, first, order, place, token,
+                                                               top, weights, sorted_weights);
+  TNX_CHECK_LAUNCH("expert order");
+  return 0;
+}
+
+// out[t] = residual[t] + sum_c scale[t, c] y[place[t * top + c]]
+extern "C" int tnx_expert_combine(const float* y, const int* place, const float* scale, const float* residual, float* out,
+                                  int tokens, int top, int width, hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && top > 0 && width > 0, "expert_combine: bad sizes");
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * width;
+  combine_kernel<<<blocks_for(total), 256, 0, stream>>>(y, residual, out, top, (size_t)width, total, place, scale);
+  TNX_CHECK_LAUNCH("expert combine");
   return 0;
 }

@@ -35,7 +35,7 @@ struct PrepareArgs {
 // Element `e` of head `head` of a normed projection, turned by the token's position. `x` points at the
 // projection's first head, `w` at its norm weight (or null), `r` is the factor of the norm.
 __device__ __forceinline__ float turned(const float* x, const float* w, float r, int head, int e, const PrepareArgs& a,
-                                        float pos) {
+                                        const float* cosines, const float* sines) {
   const int at = head * a.n + e;
   const float own = x[at] * r * (w ? w[at] : 1.f);
   if (a.freqs == nullptr || e >= 2 * a.half) return own;
@@ -52,8 +52,7 @@ __device__ __forceinline__ float turned(const float* x, const float* w, float r,
   }
   const int oat = head * a.n + other;
   const float mate = x[oat] * r * (w ? w[oat] : 1.f);
-  float s, c;
-  sincosf(pos * a.freqs[i], &s, &c);
+  const float s = sines[i], c = cosines[i];
   // the pair (u, v) becomes (u c - v s, v c + u s)
   return first ? own * c - mate * s : own * c + mate * s;
 }
@@ -61,8 +60,14 @@ __device__ __forceinline__ float turned(const float* x, const float* w, float r,
 template <typename T>
 __global__ void __launch_bounds__(256) qkv_prepare_kernel(PrepareArgs a) {
   __shared__ float scratch[4];
+  __shared__ float cosines[128], sines[128];       // of the token's angles, once for all heads
   const int t = blockIdx.x;
   const float* row = a.proj + (size_t)t * a.ld;
+  if (a.freqs != nullptr) {
+    const float pos = (float)a.positions[t];
+    for (int i = threadIdx.x; i < a.half; i += 256) sincosf(pos * a.freqs[i], &sines[i], &cosines[i]);
+  }
+  __syncthreads();
   const int nq = a.heads * a.n, nk = a.groups * a.n;
   const float* xq = row;
   const float* xk = row + nq;
@@ -78,11 +83,10 @@ __global__ void __launch_bounds__(256) qkv_prepare_kernel(PrepareArgs a) {
     s = block_sum<4>(s, scratch);
     rk = 1.f / sqrtf(s / (float)nk + a.eps);
   }
-  const float pos = (float)a.positions[t];
   T* q_out = (T*)a.q_out + (size_t)t * a.heads * a.d;
   for (int i = threadIdx.x; i < a.heads * a.d; i += 256) {
     const int head = i / a.d, e = i - head * a.d;
-    q_out[i] = from_f32<T>(e < a.n ? turned(xq, a.q_weight, rq, head, e, a, pos) * a.scale : 0.f);
+    q_out[i] = from_f32<T>(e < a.n ? turned(xq, a.q_weight, rq, head, e, a, cosines, sines) * a.scale : 0.f);
   }
   const int page = a.token_page[t], off = a.token_offset[t];
   if (page < 0 || page >= a.num_pages) return;       // the host checks that every token has a page
@@ -90,7 +94,7 @@ __global__ void __launch_bounds__(256) qkv_prepare_kernel(PrepareArgs a) {
   T* vp = (T*)a.v_pages + (size_t)page * a.page_stride;
   for (int i = threadIdx.x; i < a.groups * a.d; i += 256) {
     const int g = i / a.d, e = i - g * a.d;
-    kp[((size_t)g * a.page_size + off) * a.d + e] = from_f32<T>(e < a.n ? turned(xk, a.k_weight, rk, g, e, a, pos) : 0.f);
+    kp[((size_t)g * a.page_size + off) * a.d + e] = from_f32<T>(e < a.n ? turned(xk, a.k_weight, rk, g, e, a, cosines, sines) : 0.f);
   }
   const float lam = a.first != nullptr ? a.mix_weight[0] : 0.f;
   const float* first = a.first != nullptr ? a.first + (size_t)t * a.first_ld : nullptr;
@@ -117,7 +121,7 @@ extern "C" int tnx_qkv_prepare(const float* proj, int ld, const float* q_weight,
   TNX_REQUIRE(d >= n && d >= v, "qkv_prepare: cached heads of %d elements do not hold %d and %d", d, n, v);
   TNX_REQUIRE(ld >= heads * n + groups * (n + v), "qkv_prepare: rows of %d elements, %d needed", ld,
               heads * n + groups * (n + v));
-  TNX_REQUIRE(freqs == nullptr || 2 * half <= n, "qkv_prepare: %d turned elements in heads of %d", 2 * half, n);
+  TNX_REQUIRE(freqs == nullptr || (2 * half <= n && half <= 128), "qkv_prepare: %d turned elements in heads of %d", 2 * half, n);
   TNX_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "qkv_prepare: both norm weights or none");
   TNX_REQUIRE((first == nullptr) || (mix_weight != nullptr && first_ld >= groups * v), "qkv_prepare: blending needs its weight");
   TNX_REQUIRE(page_stride >= (long long)groups * d * page_size, "qkv_prepare: pages closer than a page's elements");

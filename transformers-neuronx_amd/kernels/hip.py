@@ -130,8 +130,11 @@ _SIGNATURES = {
         "tnx_route": [_c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
         "tnx_expert_mixture": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                               _c_int, _c_void_p],
-        "tnx_gated_activation": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                               _c_int, _c_int, _c_void_p],
+        "tnx_gated_activation": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
+        "tnx_expert_order": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                             _c_void_p, _c_void_p],
+        "tnx_expert_combine": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     },
     "probe": {
         "tnx_probe_stream_read": [_c_void_p, ctypes.c_size_t, _c_void_p, _c_int, _c_void_p],
@@ -554,9 +557,11 @@ class HipOps:
                 taken += size
         return taken
 
-    def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False, force_tiled=False, f32_by_library=False):
+    def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False, force_tiled=False, f32_by_library=False,
+               into=None):
         """`f32_by_library`: a float32 result without a residual may come from the vendor library too (many rows);
-        left False such a product (the head's) stays on our kernel."""
+        left False such a product (the head's) stays on our kernel. `into`: where such a float32 result goes (rows
+        of a larger tensor), instead of a tensor of its own."""
         if isinstance(x, DeferredNorm):
             folded = self._folded_for(x, w) if (residual is None and not out_f32 and force_tiled != 1) else None
             if folded is not None and self._library_product(x.shape[0], w.tensor.shape[0], w.tensor.shape[1],
@@ -639,7 +644,7 @@ class HipOps:
                 self._call("elementwise", "tnx_epilogue", _ptr(y), _ptr(bias), _ACT[act], _ptr(residual), _ptr(out),
                            _code(out_dtype), m, n, _stream())
             return out
-        out = torch.empty(m, n, dtype=out_dtype, device=x.device)
+        out = torch.empty(m, n, dtype=out_dtype, device=x.device) if into is None else _want(into, "into", out_dtype, (m, n))
         if (f32_by_library and out_f32 and residual is None and act in (None, "none") and self.library_direct
                 and self._library_product(m, n, k, w, force_tiled)
                 and self._library_call(self.cast(x, torch.bfloat16), w, bias, None, out, act, m, n, k)):
@@ -1441,19 +1446,30 @@ class HipOps:
                    _ptr(chosen), _ptr(weights), _stream())
         return chosen, weights
 
-    def gated_activation(self, gate_up, activation):
+    def gated_activation(self, gate_up, activation, row_weights=None):
         """See `ReferenceOps.gated_activation`."""
         _want(gate_up, "gate and up", torch.float32)
         t, two_f = gate_up.shape
         if two_f % 2 or activation not in _GATE_ACT:
             raise ValueError(f"gated_activation: rows of {two_f}, activation {activation!r}")
+        if row_weights is not None:
+            _want(row_weights, "row weights", torch.float32, (t,))
         out = torch.empty(t, two_f // 2, dtype=self.dtype, device=gate_up.device)
         self._call("experts", "tnx_gated_activation", _ptr(gate_up), _ptr(out), _code(self.dtype), t, two_f // 2,
-                   _GATE_ACT[activation], _stream(), work=(f"{t}x{two_f // 2}", t * two_f * 4.0 + out.numel() * out.element_size(), 0.0))
+                   _GATE_ACT[activation], _ptr(row_weights), _stream(),
+                   work=(f"{t}x{two_f // 2}", t * two_f * 4.0 + out.numel() * out.element_size(), 0.0))
         return out
 
-    def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None):
-        """See `ReferenceOps.expert_mixture`."""
+    # A step of this many (token, choice) pairs an expert or more, bfloat16, that is not being recorded: the host
+    # reads where each expert's pairs begin (one small copy that waits for the device) and every expert's two
+    # products go to the vendor library over its own rows, as the many-rows products of the other parts do. Below
+    # that, and in recorded steps, one launch of ours takes all experts and the host reads nothing. 0: never.
+    expert_library_rows = 96
+    expert_plain_products = False      # tests set it: the kernel without the matrix unit in bfloat16 too
+
+    def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None, may_wait=False):
+        """See `ReferenceOps.expert_mixture`. `may_wait`: the step is not being recorded, so the host may read
+        what the device has made."""
         t, top = chosen.shape
         experts, two_f, width = w_gate_up.shape
         f = two_f // 2
@@ -1467,15 +1483,41 @@ class HipOps:
         if residual is not None:
             _want(residual, "residual", torch.float32, (t, width))
         dev = h.device
-        ints = torch.empty(experts + 1 + t * top, dtype=torch.int32, device=dev)
-        inner = torch.empty(t * top, f, dtype=h.dtype, device=dev)
-        rows = torch.empty(t * top, width, dtype=torch.float32, device=dev) if top > 1 else None
+        pairs = t * top
         out = torch.empty(t, width, dtype=torch.float32, device=dev)
+        if (may_wait and self.expert_library_rows > 0 and pairs >= self.expert_library_rows * experts
+                and self.dtype == torch.bfloat16 and h.dtype == torch.bfloat16 and width % 8 == 0 and f % 8 == 0
+                and self.library_direct and not debug.tapping()):
+            ints = torch.empty(experts + 1 + 3 * pairs, dtype=torch.int32, device=dev)
+            first, order = ints[:experts + 1], ints[experts + 1:experts + 1 + pairs]
+            place, token = ints[experts + 1 + pairs:experts + 1 + 2 * pairs], ints[experts + 1 + 2 * pairs:]
+            sorted_weights = torch.empty(pairs, dtype=torch.float32, device=dev)
+            self._call("experts", "tnx_expert_order", _ptr(chosen), _ptr(weights), t, experts, top, _ptr(first), _ptr(order),
+                       _ptr(place), _ptr(token), _ptr(sorted_weights), _stream())
+            rows = self.gather_rows(h, token)                    # the pairs' tokens' rows, expert by expert
+            begins = first.tolist()                              # the host waits here for the device
+            y = torch.empty(pairs, width, dtype=torch.float32, device=dev)
+            on_input = weight_on == "input"
+            for e in range(experts):
+                a, b = begins[e], begins[e + 1]
+                if b == a:
+                    continue
+                gu = self.linear(rows[a:b], w_gate_up[e], None, out_f32=True, f32_by_library=True)
+                inner = self.gated_activation(gu, activation, sorted_weights[a:b] if on_input else None)
+                self.linear(inner, w_down[e], None, out_f32=True, f32_by_library=True, into=y[a:b])
+            self._call("experts", "tnx_expert_combine", _ptr(y), _ptr(place), None if on_input else _ptr(weights),
+                       _ptr(residual), _ptr(out), t, top, width, _stream(),
+                       work=(f"{t}x{top}x{width}", (pairs + 2.0 * t) * width * 4, 0.0))
+            return out
+        ints = torch.empty(experts + 1 + pairs, dtype=torch.int32, device=dev)
+        inner = torch.empty(pairs, f, dtype=h.dtype, device=dev)
+        rows = torch.empty(pairs, width, dtype=torch.float32, device=dev) if top > 1 else None
         item = h.element_size()
-        used = min(experts, t * top)
+        used = min(experts, pairs)
         self._call("experts", "tnx_expert_mixture", _ptr(h), _ptr(chosen), _ptr(weights), _ptr(w_gate_up), _ptr(w_down),
                    _ptr(ints[:experts + 1]), _ptr(ints[experts + 1:]), _ptr(inner), _ptr(rows), _ptr(residual), _ptr(out),
-                   _code(h.dtype), t, experts, top, width, f, _GATE_ACT[activation], int(weight_on == "input"), _stream(),
+                   _code(h.dtype), t, experts, top, width, f, _GATE_ACT[activation], int(weight_on == "input"),
+                   int(bool(self.expert_plain_products)), _stream(),
                    work=(f"{t}x{top} of {experts}", used * 3.0 * f * width * item + t * width * (item + 8.0),
                          6.0 * t * top * f * width))
         return out

@@ -505,13 +505,16 @@ class ReferenceOps:
             return g * torch.sigmoid(g)
         return ReferenceOps.activation(g, activation)
 
-    def gated_activation(self, gate_up, activation, weights=None):
-        """`act(g) * u` from float32 `[T, 2 F]` = [g | u], in the compute dtype."""
+    def gated_activation(self, gate_up, activation, row_weights=None):
+        """`act(g) * u` from float32 `[T, 2 F]` = [g | u], in the compute dtype; `row_weights` `[T]`: a factor a
+        row on both g and u."""
         f = gate_up.shape[1] // 2
         g, u = gate_up[:, :f].float(), gate_up[:, f:].float()
+        if row_weights is not None:
+            g, u = g * row_weights.float()[:, None], u * row_weights.float()[:, None]
         return (self._gate(g, activation) * u).to(self.dtype)
 
-    def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None):
+    def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None, may_wait=False):
         """float32 `residual + sum_c expert_(chosen[t, c])(h[t])` with the weights `weights[t, c]` on the expert's
         input (`weight_on="input"`: act(w g) * (w u), the float32 sums of the first product times w) or on its
         output. `w_gate_up` `[E, 2 F, D]` (gate rows, then up rows), `w_down` `[E, D, F]`."""

@@ -133,9 +133,11 @@ class ExpertMixture(FeedForward):
 
     def forward(self, h, ctx, residual):
         ops = self.ops
-        z = ops.linear(h, self.w_router, None, out_f32=True)
+        z = ops.linear(h, self.w_router, None, out_f32=True, f32_by_library=True)
         chosen, weights = ops.route(z, self.top, self.score, self.renormalize)
-        x = ops.expert_mixture(h, chosen, weights, self.w_gate_up, self.w_down, self.activation, self.weight_on, residual)
+        # (a step that is being recorded is sized by `length_bound`; any other may let the host read)
+        x = ops.expert_mixture(h, chosen, weights, self.w_gate_up, self.w_down, self.activation, self.weight_on, residual,
+                               may_wait=ctx is not None and ctx.length_bound is None)
         if not self.shared_inner:
             return x
         inner = ops.gated_activation(ops.linear(h, self.w_shared_in, None, out_f32=True, f32_by_library=True),
