@@ -123,7 +123,7 @@ _SIGNATURES = {
     },
     "memory": {
         "tnx_matrix_memory": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                              _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                              _c_int, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                               _c_int, _c_float, _c_void_p],
     },
     "experts": {
@@ -1424,10 +1424,11 @@ class HipOps:
         _want(normalizer, "normalizer", torch.float32, (slots, 2, h, n))
         _want(peak, "peak", torch.float32, (slots, 2, h))
         raw = torch.empty(t, h * v, dtype=torch.float32, device=proj.device)
+        gates = torch.empty(3, t, h, dtype=torch.float32, device=proj.device)     # two factors and a denominator a token
         out = torch.empty(t, h * v, dtype=self.dtype, device=proj.device)
         state = float(ctx.num_requests) * h * n * v * 8
         self._call("memory", "tnx_matrix_memory", _ptr(proj), total, _ptr(ctx.run_start), _ptr(ctx.cached_lens),
-                   _ptr(ctx.slots), _ptr(memory), _ptr(normalizer), _ptr(peak), slots, _ptr(raw), _ptr(norm_weight),
+                   _ptr(ctx.slots), _ptr(memory), _ptr(normalizer), _ptr(peak), slots, _ptr(raw), _ptr(gates), _ptr(norm_weight),
                    float(eps), _ptr(out), _code(self.dtype), t, ctx.num_requests, h, n, v, float(gate_cap), _stream(),
                    work=(f"{t} tokens {ctx.num_requests} runs", state + t * total * 4.0, 4.0 * t * h * n * v))
         return out
@@ -1465,6 +1466,7 @@ class HipOps:
     # products go to the vendor library over its own rows, as the many-rows products of the other parts do. Below
     # that, and in recorded steps, one launch of ours takes all experts and the host reads nothing. 0: never.
     expert_library_rows = 96
+    expert_row_step = 128
     expert_plain_products = False      # tests set it: the kernel without the matrix unit in bfloat16 too
 
     def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None, may_wait=False):
@@ -1488,22 +1490,29 @@ class HipOps:
         if (may_wait and self.expert_library_rows > 0 and pairs >= self.expert_library_rows * experts
                 and self.dtype == torch.bfloat16 and h.dtype == torch.bfloat16 and width % 8 == 0 and f % 8 == 0
                 and self.library_direct and not debug.tapping()):
-            ints = torch.empty(experts + 1 + 3 * pairs, dtype=torch.int32, device=dev)
+            step = self.expert_row_step
+            ints = torch.zeros(experts + 1 + 3 * pairs + step, dtype=torch.int32, device=dev)
             first, order = ints[:experts + 1], ints[experts + 1:experts + 1 + pairs]
             place, token = ints[experts + 1 + pairs:experts + 1 + 2 * pairs], ints[experts + 1 + 2 * pairs:]
-            sorted_weights = torch.empty(pairs, dtype=torch.float32, device=dev)
+            sorted_weights = torch.zeros(pairs + step, dtype=torch.float32, device=dev)      # zeros behind the pairs
             self._call("experts", "tnx_expert_order", _ptr(chosen), _ptr(weights), t, experts, top, _ptr(first), _ptr(order),
                        _ptr(place), _ptr(token), _ptr(sorted_weights), _stream())
-            rows = self.gather_rows(h, token)                    # the pairs' tokens' rows, expert by expert
-            begins = first.tolist()                              # the host waits here for the device
-            y = torch.empty(pairs, width, dtype=torch.float32, device=dev)
+            # An expert's products run over its rows filled up to a multiple of `expert_row_step`, so that the
+            # library's choice for a size is made once and found again: the rows behind an expert's own are the next
+            # expert's, whose products come later on the stream and write over what these left there.
+            step = self.expert_row_step
+            rows = self.gather_rows(h, token)                               # the pairs' tokens' rows, expert by expert
+            begins = first.tolist()                                         # the host waits here for the device
+            y = torch.empty(pairs + step, width, dtype=torch.float32, device=dev)
+            scale = sorted_weights
             on_input = weight_on == "input"
             for e in range(experts):
                 a, b = begins[e], begins[e + 1]
                 if b == a:
                     continue
+                b = a + -(-(b - a) // step) * step
                 gu = self.linear(rows[a:b], w_gate_up[e], None, out_f32=True, f32_by_library=True)
-                inner = self.gated_activation(gu, activation, sorted_weights[a:b] if on_input else None)
+                inner = self.gated_activation(gu, activation, scale[a:b] if on_input else None)
                 self.linear(inner, w_down[e], None, out_f32=True, f32_by_library=True, into=y[a:b])
             self._call("experts", "tnx_expert_combine", _ptr(y), _ptr(place), None if on_input else _ptr(weights),
                        _ptr(residual), _ptr(out), t, top, width, _stream(),
