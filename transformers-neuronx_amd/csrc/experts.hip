@@ -206,12 +206,21 @@ __global__ void __launch_bounds__(256) expert_product_kernel(ProductArgs p) {
 
 // The same tile on the matrix unit, bfloat16 with an inner size in 8s: a wave takes 16 columns (and with GATED the
 // 16 up rows that go with its 16 gate rows) for the tile's 16 pairs and makes out^T[column][pair] with MFMA
-// 16x16x32, the matrix's rows as the A operand, 16 bytes a lane as they lie and read once, the pairs' rows as the B
-// operand. Nothing goes through LDS: an expert's matrix is read once for every 16 of its pairs, which in a decode
-// step is once, and the rows of the pairs come from the caches.
+// 16x16x32, the matrix's rows as the A operand, the pairs' rows as the B operand. An expert's matrix is read once
+// for every 16 of its pairs, which in a decode step is once, so what counts is how the matrix streams: a wave
+// brings KC elements of each of its rows into a piece of LDS of its own with loads that cover a row's bytes side
+// by side (512 bytes or more a row and instruction, marked as read once), all of a chunk's loads under way
+// together, and takes the operands from there; the pairs' rows come from the caches. The waves of a block never
+// wait for one another.
 template <bool GATED>
 __global__ void __launch_bounds__(256) expert_product_mfma_kernel(ProductArgs p) {
   constexpr int TM = 16;
+  constexpr int ROWS = GATED ? 32 : 16;                   // rows of the matrix a wave holds
+  constexpr int KC = 256;                                 // elements of a row a chunk
+  constexpr int LD = KC + 8;                              // a row in LDS: 16 bytes more, so that rows lie in different banks
+  constexpr int LPR = KC / 8, RPI = 64 / LPR;             // lanes a row, rows an instruction
+  constexpr int LOADS = ROWS / RPI;
+  __shared__ __attribute__((aligned(16))) bf16_t staged[4][ROWS * LD];
   int tile = blockIdx.y, e = 0, begin = 0, end = 0;
   for (; e < p.experts; ++e) {
     begin = p.first[e];
@@ -223,27 +232,41 @@ __global__ void __launch_bounds__(256) expert_product_mfma_kernel(ProductArgs p)
   if (e >= p.experts) return;
   begin += tile * TM;
   const int count = min(TM, end - begin);
-  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
-  const int col0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 16;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+  const int col0 = (blockIdx.x * 4 + wave) * 16;
   if (col0 >= p.n) return;
   const int pair = r < count ? p.order[begin + r] : -1;
   const bf16_t* xrow = (const bf16_t*)p.a + (size_t)(pair < 0 ? 0 : (GATED ? pair / p.top : pair)) * p.k;
   const bf16_t* W = (const bf16_t*)p.w + (size_t)e * (GATED ? 2 : 1) * p.n * p.k;
-  const int n = col0 + r;
-  const bf16_t* wrow = W + (size_t)min(n, p.n - 1) * p.k;
-  const bf16_t* urow = wrow + (size_t)p.n * p.k;          // GATED: the up row of the same column
+  bf16_t* mine = staged[wave];
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  // load i of a chunk: row RPI i + lane / LPR of the wave's rows (the up rows behind the gate rows), elements 8 (lane % LPR) on
+  const int lrow = lane / LPR, lcol = 8 * (lane % LPR);
+  const bf16_t* src[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int row = RPI * i + lrow;                       // 0 .. 15 gate (or plain) rows, 16 .. 31 up rows
+    const int n = col0 + (row & 15);
+    src[i] = n < p.n ? W + ((size_t)(row >> 4) * p.n + n) * p.k + lcol : nullptr;
+  }
   f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc_up = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-  for (int k0 = 0; k0 < p.k; k0 += 32) {
-    const int d0 = k0 + 8 * g;
-    const bool in = d0 < p.k;
-    const bf16x8 b = (in && pair >= 0) ? *(const bf16x8*)(xrow + d0) : zero8;
-    const bf16x8 a = (in && n < p.n) ? load_once(wrow + d0) : zero8;
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
-    if (GATED) {
-      const bf16x8 u = (in && n < p.n) ? load_once(urow + d0) : zero8;
-      acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u, b, acc_up, 0, 0, 0);
+  for (int k0 = 0; k0 < p.k; k0 += KC) {
+    bf16x8 got[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) got[i] = (src[i] != nullptr && k0 + lcol < p.k) ? load_once(src[i] + k0) : zero8;
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) *(bf16x8*)(mine + (RPI * i + lrow) * LD + lcol) = got[i];
+    const int steps = min(KC, p.k - k0);
+    for (int kk = 0; kk < steps; kk += 32) {
+      const int d0 = kk + 8 * g;
+      const bool in = k0 + d0 < p.k;
+      const bf16x8 b = (in && pair >= 0) ? *(const bf16x8*)(xrow + k0 + d0) : zero8;
+      const bf16x8 a = *(const bf16x8*)(mine + r * LD + d0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+      if (GATED) {
+        const bf16x8 u = *(const bf16x8*)(mine + (16 + r) * LD + d0);
+        acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u, b, acc_up, 0, 0, 0);
+      }
     }
   }
   if (pair < 0) return;
@@ -265,7 +288,6 @@ __global__ void __launch_bounds__(256) expert_product_mfma_kernel(ProductArgs p)
   }
 }
 
-// out[t] = residual[t] + sum_c y[t * top + c], in the order of c
 // (`place`: the row of y that holds pair t * top + c, where the rows lie in another order; `scale`: a factor a pair)
 __global__ void combine_kernel(const float* __restrict__ y, const float* __restrict__ residual, float* __restrict__ out,
                                int top, size_t n, size_t total, const int* __restrict__ place,
