@@ -138,7 +138,7 @@ def test_matrix_memory_across_steps_cut_anywhere(name, dtype, tol, sizes):
              "p.i": eye[-2 * heads:-heads], "p.f": eye[-heads:], "p.i.b": torch.zeros(heads, dtype=F64),
              "p.f.b": torch.zeros(heads, dtype=F64), "p.norm": nw.double(), "p.o": torch.eye(hv, dtype=F64)}
         want[r] = P.mlstm(m, w, "p.", x, eps)
-    state = [torch.full((3, 2, heads, n, v), 3.0, device=DEV), torch.full((3, 2, heads, n), -2.0, device=DEV),
+    state = [torch.full((3, 2, heads, v, n), 3.0, device=DEV), torch.full((3, 2, heads, n), -2.0, device=DEV),
              torch.full((3, 2, heads), 5.0, device=DEV)]
     # request 0 in slot 2, request 1 in slot 0 from the third step on
     cuts0 = [0, 1, 2, 4, 5, 6, 30, 32, 45]

@@ -17,7 +17,7 @@ struct CellArgs {
   const int* run_start;   // [R + 1]
   const int* cached;      // [R]
   const int* slots;       // [R]
-  float* memory;          // [slots, 2, H, n, v]
+  float* memory;          // [slots, 2, H, v, n]
   float* normalizer;      // [slots, 2, H, n]
   float* peak;            // [slots, 2, H]
   float* out;             // [T, H v], before the norm
@@ -30,17 +30,22 @@ __device__ __forceinline__ float log_sigmoid(float z) {
   return fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
 }
 
-// The recurrence is taken apart. Its gates and its normalizer need nothing of S: one block a (request, head) walks
-// the run's tokens (`memory_gates_kernel`), leaves every token's two factors exp(f + m - m'), exp(i - m') and the
-// reciprocal of the denominator max(|nrm' . q|, exp(-m')) + 1e-6 in memory, and carries nrm and m on. The blocks
-// that hold S (`memory_cell_kernel`, 64 columns each) then have nothing but multiply-adds between one token and
-// the next, and no two blocks share state that either writes.
+// The recurrence is taken apart. The gates need nothing of S: one wave a (request, head) walks the run's tokens
+// (`memory_gates_kernel`), leaves every token's two factors exp(f + m - m'), exp(i - m') and the floor exp(-m') of
+// its denominator in memory, carries m on, and sets the normalizer the run begins with aside. The blocks that hold
+// S (`memory_cell_kernel`, 16 columns each) each carry the normalizer along as one more column, so that between
+// one token and the next there is nothing but multiply-adds and sums within 16 lanes, and no block reads state
+// that another writes: they read the normalizer from where the first kernel set it aside, and the block of a
+// head's first columns alone writes it back.
 //
-// Both take a run a chunk of tokens at a time through LDS. A token's queries, keys and values lie far from the
-// next token's (a row of all heads' projections apart), so what counts is how many loads are under way: every
-// thread loads 16 bytes at a time into registers, the next chunk's while this chunk is worked on, and the
-// registers go to LDS afterwards. ALIGNED: rows and heads begin at multiples of 16 bytes; otherwise the same with
-// loads of one element.
+// The state lies with a column's rows side by side (`memory` [slots, 2, H, v, n]): a lane's rows of a column are
+// neighbours in memory.
+//
+// A run goes a chunk of tokens at a time through LDS. A token's queries, keys and values lie far from the next
+// token's (a row of all heads' projections apart), so what counts is how many loads are under way: every thread
+// loads 16 bytes at a time into registers, the next chunk's while this chunk is worked on, and the registers go to
+// LDS afterwards. ALIGNED: rows and heads begin at multiples of 16 bytes; otherwise the same with loads of one
+// element.
 
 template <bool ALIGNED>
 __device__ __forceinline__ f32x4 load4(const float* p, int valid) {      // the first `valid` of four elements, zeros behind
@@ -53,197 +58,133 @@ __device__ __forceinline__ f32x4 load4(const float* p, int valid) {      // the 
   return r;
 }
 
-// grid: requests * heads blocks of four waves. All threads load; the first wave walks the chain, a row of the
-// normalizer a lane (and up to four). LDS: [CHG][np + 1] queries (scaled) and keys, 8 numbers a token.
-constexpr int CHG = 32;      // the most tokens a chunk; `chg` of them where LDS holds no more
-template <bool ALIGNED>
-__global__ void __launch_bounds__(256) memory_gates_kernel(CellArgs a, float* __restrict__ keeps, float* __restrict__ takes,
-                                                           float* __restrict__ belows, int np, int chg) {
-  extern __shared__ float lds[];
+// grid: requests * heads blocks of one wave; 64 tokens a round, a token a lane, the running maximum a chain of
+// lane 0 between two rounds of side-by-side work.
+__global__ void __launch_bounds__(64) memory_gates_kernel(CellArgs a, float* __restrict__ keeps, float* __restrict__ takes,
+                                                          float* __restrict__ floors, float* __restrict__ aside) {
+  __shared__ float gis[64], gfs[64], ms[65];
   const int r = blockIdx.x / a.heads, head = blockIdx.x - r * a.heads;
   const int lane = threadIdx.x;
   const int start = a.run_start[r], count = a.run_start[r + 1] - start;
   const int have = a.cached[r], slot = a.slots[r];
   const int hn = a.heads * a.n, hv = a.heads * a.v;
   if (count <= 0) return;
-  const int ldq = np + 1;                           // a token's row in LDS: one more, so that tokens lie in different banks
-  float* qs = lds;                                  // [CHG][ldq]
-  float* ks = qs + chg * ldq;                       // [CHG][ldq]
-  float* gis = ks + chg * ldq;                      // [CHG] log of the input gate
-  float* gfs = gis + chg;                           // [CHG] log of the forget gate
-  float* ms = gfs + chg;                            // [CHG + 1] the running maximum
-  float* kp = ms + chg + 1;                         // [CHG] exp(f + m - m')
-  float* tk = kp + chg;                             // [CHG] exp(i - m')
-  float* fl = tk + chg;                             // [CHG] exp(-m')
   const int from = (have - 1) & 1, to = (have + count - 1) & 1;
   const size_t head_at = (size_t)slot * 2 * a.heads + head;
-  float nrm[4] = {0.f, 0.f, 0.f, 0.f}, m = 0.f;     // lane l of the first wave holds rows l, l + 64, l + 128, l + 192
-  if (lane < 64) {
+  {
     const float* np_ = a.normalizer + (head_at + (size_t)from * a.heads) * a.n;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) nrm[j] = (have > 0 && lane + 64 * j < a.n) ? np_[lane + 64 * j] : 0.f;
-    if (have > 0) m = a.peak[head_at + (size_t)from * a.heads];
+    float* out = aside + (size_t)blockIdx.x * a.n;
+    for (int d = lane; d < a.n; d += 64) out[d] = have > 0 ? np_[d] : 0.f;
   }
-  const int fours = np >> 2;                        // 16-byte pieces of a token's queries: up to 64
-  f32x4 rq[8], rk[8];                               // CHG * fours / 256 <= 8 pieces a thread
-  float ri = 0.f, rf = 0.f;
-  auto fetch = [&](int t0) {
-    const int len = min(chg, count - t0);
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int f = lane + 256 * u, t = f / fours, d = 4 * (f - t * fours);
-      const bool in = f < chg * fours && t < len;
-      const float* row = a.proj + (size_t)(start + t0 + (in ? t : 0)) * a.ld + head * a.n + d;
-      rq[u] = load4<ALIGNED>(row, in ? a.n - d : 0);
-      rk[u] = load4<ALIGNED>(row + hn, in ? a.n - d : 0);
-    }
+  float m = have > 0 ? a.peak[head_at + (size_t)from * a.heads] : 0.f;
+  for (int t0 = 0; t0 < count; t0 += 64) {
+    const int len = min(64, count - t0);
     if (lane < len) {
       const float* row = a.proj + (size_t)(start + t0 + lane) * a.ld + 2 * hn + 2 * hv;
-      ri = row[head];
-      rf = row[a.heads + head];
+      gis[lane] = a.cap * tanhf(row[head] / a.cap);
+      gfs[lane] = log_sigmoid(a.cap * tanhf(row[a.heads + head] / a.cap));
     }
-  };
-  auto stash = [&](int t0) {
-    const int len = min(chg, count - t0);
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int f = lane + 256 * u, t = f / fours, d = 4 * (f - t * fours);
-      if (f < chg * fours) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) qs[t * ldq + d + e] = rq[u][e] * a.q_scale, ks[t * ldq + d + e] = rk[u][e];
-      }
-    }
-    if (lane < len) {
-      gis[lane] = a.cap * tanhf(ri / a.cap);
-      gfs[lane] = log_sigmoid(a.cap * tanhf(rf / a.cap));
-    }
-  };
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  for (int t0 = 0; t0 < count; t0 += chg) {
-    const int len = min(chg, count - t0);
-    const bool more = t0 + chg < count;
-    if (more) fetch(t0 + chg);                      // under way while this chunk is worked on
+    __syncthreads();
     if (lane == 0) {
+      // (what the chain reads from LDS is read before it begins: a store into LDS between two loads would keep the
+      // second load from being under way with the first)
+      float gi_r[64], gf_r[64], after[64], peak = m;
+#pragma unroll
+      for (int t = 0; t < 64; ++t) gi_r[t] = t < len ? gis[t] : 0.f, gf_r[t] = t < len ? gfs[t] : 0.f;
+#pragma unroll
+      for (int t = 0; t < 64; ++t) after[t] = peak = t < len ? fmaxf(gf_r[t] + peak, gi_r[t]) : peak;
       ms[0] = m;                                    // ms[t + 1]: the maximum after token t
-      for (int t = 0; t < len; ++t) ms[t + 1] = m = fmaxf(gfs[t] + m, gis[t]);
+#pragma unroll
+      for (int t = 0; t < 64; ++t)
+        if (t < len) ms[t + 1] = after[t];
     }
     __syncthreads();
     if (lane < len) {
       const size_t at = (size_t)(start + t0 + lane) * a.heads + head;
-      keeps[at] = kp[lane] = expf(gfs[lane] + ms[lane] - ms[lane + 1]);
-      takes[at] = tk[lane] = expf(gis[lane] - ms[lane + 1]);
-      fl[lane] = expf(-ms[lane + 1]);
+      keeps[at] = expf(gfs[lane] + ms[lane] - ms[lane + 1]);
+      takes[at] = expf(gis[lane] - ms[lane + 1]);
+      floors[at] = expf(-ms[lane + 1]);
     }
+    m = ms[len];
     __syncthreads();
-    // the normalizer's chain, a row a lane: its products with the queries take the queries' places, and the
-    // tokens' sums over the rows are then made side by side, a token a lane
-    if (lane < 64) {
-#pragma unroll 4
-      for (int t = 0; t < len; ++t) {
-        const float keep = kp[t], take = tk[t];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int d = lane + 64 * j;
-          if (d < np) {
-            nrm[j] = keep * nrm[j] + take * ks[t * ldq + d];
-            qs[t * ldq + d] *= nrm[j];
-          }
-        }
-      }
-    }
-    __syncthreads();
-    if (lane < len) {
-      float dot = 0.f;
-      for (int d = 0; d < np; ++d) dot += qs[lane * ldq + d];
-      belows[(size_t)(start + t0 + lane) * a.heads + head] = 1.f / (fmaxf(fabsf(dot), fl[lane]) + 1e-6f);
-    }
-    __syncthreads();
-    if (more) {
-      stash(t0 + chg);
-      __syncthreads();
-    }
-  }
-  if (lane < 64) {
-    float* np_ = a.normalizer + (head_at + (size_t)to * a.heads) * a.n;
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (lane + 64 * j < a.n) np_[lane + 64 * j] = nrm[j];
   }
   if (lane == 0) a.peak[head_at + (size_t)to * a.heads] = m;
 }
 
-// grid: requests * heads * column blocks; a block is four waves and 64 columns of S: wave w holds the columns
-// 64 b + 16 w + (lane & 15), and of these the rows NR (lane >> 4) + j, j < NR: a lane's share of a column is a
-// quarter of its rows, and the four quarters meet through the wave's row exchanges (`rows_sum`).
+// grid: requests * heads * column blocks; a block is four waves and 16 columns of S. In a wave the 16 lanes of a
+// row of lanes share a column (column 16 b + 4 w + lane / 16): lane % 16 holds its rows NR (lane % 16) + j, j < NR,
+// and the same rows of the normalizer; a column's sum over the rows is a sum over the 16 lanes of a row of lanes.
 template <int NR, bool ALIGNED>
 __global__ void __launch_bounds__(256) memory_cell_kernel(CellArgs a, const float* __restrict__ keeps,
                                                           const float* __restrict__ takes,
-                                                          const float* __restrict__ belows, int column_blocks) {
-  constexpr int CH = NR == 64 ? 16 : 32;                  // tokens a chunk
-  constexpr int np = 4 * NR;                              // a token's queries (and keys) in LDS, zeros behind n
-  constexpr int QN = CH * NR / 256;                       // 16-byte pieces of queries (and keys) a thread and chunk
-  constexpr int VN = CH * 16 / 256;                       // and of values
+                                                          const float* __restrict__ floors,
+                                                          const float* __restrict__ aside, int column_blocks) {
+  constexpr int CH = NR == 16 ? 16 : 32;                  // tokens a chunk
+  constexpr int np = 16 * NR;                             // a token's queries (and keys) in LDS, zeros behind n
+  constexpr int PT = np / 4;                              // 16-byte pieces of a token's queries
+  constexpr int QN = (CH * PT + 255) / 256;               // pieces of queries (and keys) a thread and chunk
   __shared__ __attribute__((aligned(16))) float qs[CH * np];      // queries, scaled
   __shared__ __attribute__((aligned(16))) float ks[CH * np];      // keys times exp(i - m')
-  __shared__ __attribute__((aligned(16))) float vs[CH * 64];
-  __shared__ float kp[CH], bl[CH];                        // exp(f + m - m'), one over the denominators
+  __shared__ __attribute__((aligned(16))) float vs[CH * 16];
+  __shared__ float kp[CH], fl[CH];                        // exp(f + m - m'), exp(-m')
   const int cb = blockIdx.x % column_blocks, rh = blockIdx.x / column_blocks;
   const int r = rh / a.heads, head = rh - r * a.heads;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int quarter = lane >> 4;
+  const int grp = lane & 15;
   const int start = a.run_start[r], count = a.run_start[r + 1] - start;
   const int have = a.cached[r], slot = a.slots[r];
   const int hn = a.heads * a.n, hv = a.heads * a.v;
   if (count <= 0) return;
-  const int col = 64 * cb + 16 * wave + (lane & 15);
+  const int col = 16 * cb + 4 * wave + (lane >> 4);
   const bool col_ok = col < a.v;
-  float S[NR];
+  float S[NR], nrm[NR];
   const int from = (have - 1) & 1, to = (have + count - 1) & 1;
   const size_t head_at = (size_t)slot * 2 * a.heads + head;        // + place * heads
   {
-    const float* Sp = a.memory + (head_at + (size_t)from * a.heads) * a.n * a.v;
+    const float* Sp = a.memory + ((head_at + (size_t)from * a.heads) * a.v + (col_ok ? col : 0)) * a.n;
+    const float* np_ = aside + (size_t)rh * a.n;
 #pragma unroll
     for (int j = 0; j < NR; ++j) {
-      const int d = quarter * NR + j;
-      S[j] = (have > 0 && d < a.n && col_ok) ? Sp[(size_t)d * a.v + col] : 0.f;
+      const int d = grp * NR + j;
+      S[j] = (have > 0 && d < a.n && col_ok) ? Sp[d] : 0.f;
+      nrm[j] = d < a.n ? np_[d] : 0.f;
     }
   }
-  f32x4 rq[QN], rk[QN], rv[VN];
-  float rt[QN], rkeep = 0.f, rbl = 0.f;
+  f32x4 rq[QN], rk[QN], rv = {0.f, 0.f, 0.f, 0.f};
+  float rt[QN], rkeep = 1.f, rfl = 0.f;
   auto fetch = [&](int t0) {
     const int len = min(CH, count - t0);
 #pragma unroll
     for (int u = 0; u < QN; ++u) {
-      const int f = threadIdx.x + 256 * u, t = f / NR, d = 4 * (f - t * NR);
-      const bool in = t < len;
+      const int f = threadIdx.x + 256 * u, t = f / PT, d = 4 * (f - t * PT);
+      const bool in = f < CH * PT && t < len;
       const float* row = a.proj + (size_t)(start + t0 + (in ? t : 0)) * a.ld + head * a.n + d;
       rq[u] = load4<ALIGNED>(row, in ? a.n - d : 0);
       rk[u] = load4<ALIGNED>(row + hn, in ? a.n - d : 0);
       rt[u] = in ? takes[(size_t)(start + t0 + t) * a.heads + head] : 0.f;
     }
-#pragma unroll
-    for (int u = 0; u < VN; ++u) {
-      const int f = threadIdx.x + 256 * u, t = f >> 4, c = 64 * cb + 4 * (f & 15);
+    if (threadIdx.x < CH * 4) {                            // a token's 16 values: four pieces
+      const int t = threadIdx.x >> 2, c = 16 * cb + 4 * (threadIdx.x & 3);
       const bool in = t < len;
-      rv[u] = load4<ALIGNED>(a.proj + (size_t)(start + t0 + (in ? t : 0)) * a.ld + 2 * hn + head * a.v + c, in ? a.v - c : 0);
+      rv = load4<ALIGNED>(a.proj + (size_t)(start + t0 + (in ? t : 0)) * a.ld + 2 * hn + head * a.v + c, in ? a.v - c : 0);
     }
-    if (threadIdx.x < len) {
-      rkeep = keeps[(size_t)(start + t0 + threadIdx.x) * a.heads + head];
-      rbl = belows[(size_t)(start + t0 + threadIdx.x) * a.heads + head];
+    if (threadIdx.x < CH) {
+      const bool in = threadIdx.x < len;
+      rkeep = in ? keeps[(size_t)(start + t0 + threadIdx.x) * a.heads + head] : 1.f;
+      rfl = in ? floors[(size_t)(start + t0 + threadIdx.x) * a.heads + head] : 1.f;
     }
   };
   auto stash = [&]() {
 #pragma unroll
     for (int u = 0; u < QN; ++u) {
-      const int f = threadIdx.x + 256 * u;
-      *(f32x4*)(qs + 4 * f) = rq[u] * a.q_scale;          // piece f of the chunk: token f / NR, elements 4 (f % NR) on
-      *(f32x4*)(ks + 4 * f) = rk[u] * rt[u];
+      const int f = threadIdx.x + 256 * u;                // piece f of the chunk: token f / PT, elements 4 (f % PT) on
+      if (f < CH * PT) {
+        *(f32x4*)(qs + 4 * f) = rq[u] * a.q_scale;
+        *(f32x4*)(ks + 4 * f) = rk[u] * rt[u];
+      }
     }
-#pragma unroll
-    for (int u = 0; u < VN; ++u) *(f32x4*)(vs + 4 * (threadIdx.x + 256 * u)) = rv[u];
-    if (threadIdx.x < CH) kp[threadIdx.x] = rkeep, bl[threadIdx.x] = rbl;
+    if (threadIdx.x < CH * 4) *(f32x4*)(vs + 4 * threadIdx.x) = rv;
+    if (threadIdx.x < CH) kp[threadIdx.x] = rkeep, fl[threadIdx.x] = rfl;
   };
   fetch(0);
   stash();
@@ -252,22 +193,33 @@ __global__ void __launch_bounds__(256) memory_cell_kernel(CellArgs a, const floa
     const int len = min(CH, count - t0);
     const bool more = t0 + CH < count;
     if (more) fetch(t0 + CH);                             // under way while this chunk is worked on
-#pragma unroll 4
-    for (int t = 0; t < len; ++t) {
+    auto token = [&](int t) {
       const float keep = kp[t];
-      const float* q = qs + t * np + quarter * NR;
-      const float* k = ks + t * np + quarter * NR;
-      const float val = vs[t * 64 + 16 * wave + (lane & 15)];
-      float top = 0.f, top2 = 0.f;
+      const float* q = qs + t * np + grp * NR;
+      const float* k = ks + t * np + grp * NR;
+      const float val = vs[t * 16 + 4 * wave + (lane >> 4)];
+      float top = 0.f, dot = 0.f;
 #pragma unroll
-      for (int j = 0; j < NR; j += 2) {
+      for (int j = 0; j < NR; ++j) {
         S[j] = keep * S[j] + k[j] * val;
-        S[j + 1] = keep * S[j + 1] + k[j + 1] * val;
+        nrm[j] = keep * nrm[j] + k[j];
         top += S[j] * q[j];
-        top2 += S[j + 1] * q[j + 1];
+        dot += nrm[j] * q[j];
       }
-      const float o = rows_sum(top + top2) * bl[t];
-      if (quarter == 0 && col_ok) a.out[(size_t)(start + t0 + t) * hv + head * a.v + col] = o;
+      // sums over the 16 lanes of a row of lanes
+      top += lane_dpp<TNX_DPP_XOR1>(top), dot += lane_dpp<TNX_DPP_XOR1>(dot);
+      top += lane_dpp<TNX_DPP_XOR2>(top), dot += lane_dpp<TNX_DPP_XOR2>(dot);
+      top += lane_dpp<TNX_DPP_HALF_MIRROR>(top), dot += lane_dpp<TNX_DPP_HALF_MIRROR>(dot);
+      top += lane_dpp<TNX_DPP_MIRROR>(top), dot += lane_dpp<TNX_DPP_MIRROR>(dot);
+      // (the denominator is 1e-6 at least: its reciprocal, right to a unit in the last place, is no subnormal)
+      const float o = top * __builtin_amdgcn_rcpf(fmaxf(fabsf(dot), fl[t]) + 1e-6f);
+      if (grp == 0 && col_ok) a.out[(size_t)(start + t0 + t) * hv + head * a.v + col] = o;
+    };
+    if (len == CH) {        // a whole chunk: a count the compiler knows, so that the next tokens' operands are on their way
+#pragma unroll 4
+      for (int t = 0; t < CH; ++t) token(t);
+    } else {
+      for (int t = 0; t < len; ++t) token(t);
     }
     __syncthreads();        // before the next chunk takes the place of what this one read
     if (more) {
@@ -275,11 +227,17 @@ __global__ void __launch_bounds__(256) memory_cell_kernel(CellArgs a, const floa
       __syncthreads();
     }
   }
-  float* Sp = a.memory + (head_at + (size_t)to * a.heads) * a.n * a.v;
+  if (col_ok) {
+    float* Sp = a.memory + ((head_at + (size_t)to * a.heads) * a.v + col) * a.n;
 #pragma unroll
-  for (int j = 0; j < NR; ++j) {
-    const int d = quarter * NR + j;
-    if (d < a.n && col_ok) Sp[(size_t)d * a.v + col] = S[j];
+    for (int j = 0; j < NR; ++j)
+      if (grp * NR + j < a.n) Sp[grp * NR + j] = S[j];
+  }
+  if (cb == 0 && wave == 0 && lane < 16) {                 // the normalizer, once a head
+    float* np_ = a.normalizer + (head_at + (size_t)to * a.heads) * a.n;
+#pragma unroll
+    for (int j = 0; j < NR; ++j)
+      if (grp * NR + j < a.n) np_[grp * NR + j] = nrm[j];
   }
 }
 
@@ -305,14 +263,14 @@ __global__ void __launch_bounds__(256) memory_output_kernel(const float* __restr
 }
 
 template <int NR>
-void launch_cell(const CellArgs& a, const float* keeps, const float* takes, const float* belows, int requests, bool aligned,
-                 hipStream_t stream) {
-  const int column_blocks = (a.v + 63) / 64;
+void launch_cell(const CellArgs& a, const float* keeps, const float* takes, const float* floors, const float* aside,
+                 int requests, bool aligned, hipStream_t stream) {
+  const int column_blocks = (a.v + 15) / 16;
   const dim3 grid(requests * a.heads * column_blocks);
   if (aligned)
-    memory_cell_kernel<NR, true><<<grid, 256, 0, stream>>>(a, keeps, takes, belows, column_blocks);
+    memory_cell_kernel<NR, true><<<grid, 256, 0, stream>>>(a, keeps, takes, floors, aside, column_blocks);
   else
-    memory_cell_kernel<NR, false><<<grid, 256, 0, stream>>>(a, keeps, takes, belows, column_blocks);
+    memory_cell_kernel<NR, false><<<grid, 256, 0, stream>>>(a, keeps, takes, floors, aside, column_blocks);
 }
 
 }  // namespace
@@ -331,28 +289,21 @@ extern "C" int tnx_matrix_memory(const float* proj, int ld, const int* run_start
   CellArgs a{proj, ld, run_start, cached, slots, memory, normalizer, peak, raw, heads, n, v, cap, 1.f / sqrtf((float)n)};
   float* keeps = gates;                             // [T, H] each
   float* takes = gates + (size_t)tokens * heads;
-  float* belows = gates + 2 * (size_t)tokens * heads;
+  float* floors = gates + 2 * (size_t)tokens * heads;
+  float* aside = gates + 3 * (size_t)tokens * heads;      // [R, H, n]: the normalizers the runs begin with
   // rows and heads that begin at multiples of 16 bytes are loaded 16 bytes at a time
   const bool aligned = n % 4 == 0 && v % 4 == 0 && ld % 4 == 0 && (uintptr_t)proj % 16 == 0;
-  {
-    const int np = (n + 3) / 4 * 4;
-    const int chg = np > 240 ? CHG / 2 : CHG;          // 64 KB of LDS hold 32 tokens of up to 240 elements
-    const size_t lds = ((size_t)chg * (2 * (np + 1) + 6) + 1) * sizeof(float);
-    if (aligned)
-      memory_gates_kernel<true><<<requests * heads, 256, lds, stream>>>(a, keeps, takes, belows, np, chg);
-    else
-      memory_gates_kernel<false><<<requests * heads, 256, lds, stream>>>(a, keeps, takes, belows, np, chg);
-    TNX_CHECK_LAUNCH("matrix_memory gates");
-  }
-  const int quarter_rows = (n + 3) / 4;
-  if (quarter_rows <= 8)
-    launch_cell<8>(a, keeps, takes, belows, requests, aligned, stream);
-  else if (quarter_rows <= 16)
-    launch_cell<16>(a, keeps, takes, belows, requests, aligned, stream);
-  else if (quarter_rows <= 32)
-    launch_cell<32>(a, keeps, takes, belows, requests, aligned, stream);
+  memory_gates_kernel<<<requests * heads, 64, 0, stream>>>(a, keeps, takes, floors, aside);
+  TNX_CHECK_LAUNCH("matrix_memory gates");
+  const int rows16 = (n + 15) / 16;
+  if (rows16 <= 2)
+    launch_cell<2>(a, keeps, takes, floors, aside, requests, aligned, stream);
+  else if (rows16 <= 4)
+    launch_cell<4>(a, keeps, takes, floors, aside, requests, aligned, stream);
+  else if (rows16 <= 8)
+    launch_cell<8>(a, keeps, takes, floors, aside, requests, aligned, stream);
   else
-    launch_cell<64>(a, keeps, takes, belows, requests, aligned, stream);
+    launch_cell<16>(a, keeps, takes, floors, aside, requests, aligned, stream);
   TNX_CHECK_LAUNCH("matrix_memory");
   const int pairs = tokens * heads;
   const int gate_at = 2 * heads * n + heads * v;

@@ -1420,11 +1420,12 @@ class HipOps:
         _want(proj, "projections", torch.float32, (t, total))
         _want(norm_weight, "norm weight", torch.float32, (h * v,))
         slots = memory.shape[0]
-        _want(memory, "memory", torch.float32, (slots, 2, h, n, v))
+        _want(memory, "memory", torch.float32, (slots, 2, h, v, n))
         _want(normalizer, "normalizer", torch.float32, (slots, 2, h, n))
         _want(peak, "peak", torch.float32, (slots, 2, h))
         raw = torch.empty(t, h * v, dtype=torch.float32, device=proj.device)
-        gates = torch.empty(3, t, h, dtype=torch.float32, device=proj.device)     # two factors and a denominator a token
+        # two factors and a floor a token, and the normalizer every run begins with
+        gates = torch.empty(3 * t * h + ctx.num_requests * h * n, dtype=torch.float32, device=proj.device)
         out = torch.empty(t, h * v, dtype=self.dtype, device=proj.device)
         state = float(ctx.num_requests) * h * n * v * 8
         self._call("memory", "tnx_matrix_memory", _ptr(proj), total, _ptr(ctx.run_start), _ptr(ctx.cached_lens),

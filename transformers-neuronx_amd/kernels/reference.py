@@ -449,7 +449,8 @@ class ReferenceOps:
         """The recurrence of the matrix-memory mixer over a step's runs and what follows it up to the output
         projection. `proj` float32 `[T, 2 H n + 2 H v + 2 H]`: queries, keys, values, output gates, and a head's
         input and forget pre-activations (bias added). State float32, in two places by the parity of the
-        position: `memory` `[slots, 2, H, n, v]`, `normalizer` `[slots, 2, H, n]`, `peak` `[slots, 2, H]`; the token
+        position: `memory` `[slots, 2, H, v, n]` (a column's rows side by side), `normalizer` `[slots, 2, H, n]`, `peak`
+        `[slots, 2, H]`; the token
         at position p reads place (p - 1) & 1 (nothing at p = 0: all zeros) and writes place p & 1. Returns
         `[T, H v]` in the compute dtype: each head's result at unit root mean square, weighted, times
         sigmoid(gate)."""
@@ -468,9 +469,10 @@ class ReferenceOps:
             count, slot, have = int(ctx.run_lens_host[r]), int(ctx.slots_host[r]), int(ctx.cached_lens_host[r])
             if have > 0:
                 at = (have - 1) & 1
-                mem, nrm, pk = memory[slot, at].clone(), normalizer[slot, at].clone(), peak[slot, at].clone()
+                mem, nrm, pk = memory[slot, at].transpose(1, 2).clone(), normalizer[slot, at].clone(), peak[slot, at].clone()
             else:
-                mem, nrm, pk = torch.zeros_like(memory[slot, 0]), torch.zeros_like(normalizer[slot, 0]), torch.zeros_like(peak[slot, 0])
+                mem = torch.zeros_like(memory[slot, 0]).transpose(1, 2).clone()
+                nrm, pk = torch.zeros_like(normalizer[slot, 0]), torch.zeros_like(peak[slot, 0])
             for i in range(start, start + count):
                 new = torch.maximum(gf[i] + pk, gi[i])
                 keep, take = torch.exp(gf[i] + pk - new), torch.exp(gi[i] - new)
@@ -480,7 +482,7 @@ class ReferenceOps:
                 below = torch.maximum((nrm * q[i]).sum(-1).abs(), torch.exp(-pk)) + 1e-6
                 out[i] = torch.einsum("hnv,hn->hv", mem, q[i]) / below[:, None]
             at = (have + count - 1) & 1
-            memory[slot, at], normalizer[slot, at], peak[slot, at] = mem, nrm, pk
+            memory[slot, at], normalizer[slot, at], peak[slot, at] = mem.transpose(1, 2), nrm, pk
             start += count
         out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps)
         y = out.reshape(t, h * v) * norm_weight.float() * torch.sigmoid(gate)

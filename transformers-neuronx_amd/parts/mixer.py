@@ -366,7 +366,8 @@ class MatrixMemory(Mixer):
 
     def cache_need(self) -> Optional[CacheNeed]:
         h, n, v = self.num_heads, self.head_size, self.value_size
-        return CacheNeed("state", state_shapes=(("memory", (2, h, n, v)), ("normalizer", (2, h, n)), ("peak", (2, h))))
+        # (a column's rows side by side: what a lane of the kernel holds are neighbours in memory)
+        return CacheNeed("state", state_shapes=(("memory", (2, h, v, n)), ("normalizer", (2, h, n)), ("peak", (2, h))))
 
     def _rows(self):
         h, n, v = self.num_heads, self.head_size, self.value_size
