@@ -197,6 +197,40 @@ def test_router_and_experts(name, dtype, tol, sizes):
     _close(got.cpu()[clear], want[clear], tol)
 
 
+@pytest.mark.parametrize("weight_on,score,renormalize", [("input", "sigmoid", False), ("output", "softmax", True)])
+@pytest.mark.parametrize("forced", [None, "ours", "plain"])
+def test_experts_of_a_step_of_many_tokens(weight_on, score, renormalize, forced):
+    """Many pairs an expert: the experts' products go to the vendor library over rows in expert order (the host
+    reads where each expert's rows begin); `forced`: the same step held on our own kernels, with and without the
+    matrix unit. All against sums made token by token, with the router's own choice."""
+    from transformers_neuronx_amd.parts.feed_forward import ExpertMixture
+    tokens, experts, top, width, inner = 700, 4, 2, 128, 72
+    ops = _ops(torch.bfloat16)
+    ops.expert_library_rows = 0 if forced else 96
+    ops.expert_plain_products = forced == "plain"
+    g = torch.Generator().manual_seed(6)
+    part = ExpertMixture(width, experts, top, inner, "router", "e{}.", ("gate", "up", "down"), score=score,
+                         renormalize=renormalize, weight_on=weight_on)
+    w = {d.name: (torch.randn(d.shape, generator=g) * (1.5 / d.shape[1] ** 0.5)).to(torch.bfloat16) for d in part.param_decls("p.")}
+    part.load({k: v.to(DEV) for k, v in w.items()}, "p.", ops, torch.bfloat16)
+    h = torch.randn(tokens, width, generator=g).to(torch.bfloat16)
+    residual = torch.randn(tokens, width, generator=g)
+    ctx = _ctx([tokens], [0], [0])
+    got = part.forward(h.to(DEV), ctx, residual.to(DEV))
+    chosen, weights = ops.route(ops.linear(h.to(DEV), part.w_router, None, out_f32=True), top, score, renormalize)
+    chosen, weights = chosen.cpu(), weights.cpu().double()
+    wide = P.widen(w)
+    want = residual.double().clone()
+    for t in range(tokens):
+        for c in range(top):
+            e, s = int(chosen[t, c]), weights[t, c]
+            if weight_on == "input":
+                want[t] += P.gated_expert(wide, f"p.e{e}.", s * h[t].double())
+            else:
+                want[t] += s * P.gated_expert(wide, f"p.e{e}.", h[t].double())
+    _close(got, want, 1.2e-2)
+
+
 def _standout(dtype, heads, groups, n, v, d, window, length, run, ps, standout, seed):
     """A request of `length` tokens whose last `run` are the step's: projections such that for the last query the
     key at position `standout` scores far above the rest in every head. Returns the projections of all tokens

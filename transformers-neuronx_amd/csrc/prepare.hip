@@ -57,55 +57,61 @@ __device__ __forceinline__ float turned(const float* x, const float* w, float r,
   return first ? own * c - mate * s : own * c + mate * s;
 }
 
+// grid: (tokens, 3): a block takes a token's queries, its keys or its values; each of the three needs nothing of
+// the other two.
 template <typename T>
 __global__ void __launch_bounds__(256) qkv_prepare_kernel(PrepareArgs a) {
   __shared__ float scratch[4];
   __shared__ float cosines[128], sines[128];       // of the token's angles, once for all heads
-  const int t = blockIdx.x;
+  const int t = blockIdx.x, part = blockIdx.y;
   const float* row = a.proj + (size_t)t * a.ld;
+  const int nq = a.heads * a.n, nk = a.groups * a.n;
+  const int page = a.token_page[t], off = a.token_offset[t];
+  if (part > 0 && (page < 0 || page >= a.num_pages)) return;       // the host checks that every token has a page
+  if (part == 2) {
+    const float* xv = row + nq + nk;
+    T* vp = (T*)a.v_pages + (size_t)page * a.page_stride;
+    const float lam = a.first != nullptr ? a.mix_weight[0] : 0.f;
+    const float* first = a.first != nullptr ? a.first + (size_t)t * a.first_ld : nullptr;
+    for (int i = threadIdx.x; i < a.groups * a.d; i += 256) {
+      const int g = i / a.d, e = i - g * a.d;
+      float val = 0.f;
+      if (e < a.v) {
+        val = xv[g * a.v + e];
+        if (first != nullptr) val = (1.f - lam) * val + lam * first[g * a.v + e];
+      }
+      vp[((size_t)g * a.d + e) * a.page_size + off] = from_f32<T>(val);
+    }
+    return;
+  }
   if (a.freqs != nullptr) {
     const float pos = (float)a.positions[t];
     for (int i = threadIdx.x; i < a.half; i += 256) sincosf(pos * a.freqs[i], &sines[i], &cosines[i]);
   }
-  __syncthreads();
-  const int nq = a.heads * a.n, nk = a.groups * a.n;
-  const float* xq = row;
-  const float* xk = row + nq;
-  const float* xv = row + nq + nk;
-  float rq = 1.f, rk = 1.f;
-  if (a.q_weight != nullptr) {
+  // queries (part 0) or keys (part 1): the norm over the whole projection, then head by head
+  const float* x = part == 0 ? row : row + nq;
+  const float* w = part == 0 ? a.q_weight : a.k_weight;
+  const int count = part == 0 ? nq : nk, heads = part == 0 ? a.heads : a.groups;
+  float norm = 1.f;
+  if (w != nullptr) {
     float s = 0.f;
-    for (int i = threadIdx.x; i < nq; i += 256) s += xq[i] * xq[i];
+    for (int i = threadIdx.x; i < count; i += 256) s += x[i] * x[i];
     s = block_sum<4>(s, scratch);
-    rq = 1.f / sqrtf(s / (float)nq + a.eps);
-    s = 0.f;
-    for (int i = threadIdx.x; i < nk; i += 256) s += xk[i] * xk[i];
-    s = block_sum<4>(s, scratch);
-    rk = 1.f / sqrtf(s / (float)nk + a.eps);
+    norm = 1.f / sqrtf(s / (float)count + a.eps);
   }
-  T* q_out = (T*)a.q_out + (size_t)t * a.heads * a.d;
-  for (int i = threadIdx.x; i < a.heads * a.d; i += 256) {
-    const int head = i / a.d, e = i - head * a.d;
-    q_out[i] = from_f32<T>(e < a.n ? turned(xq, a.q_weight, rq, head, e, a, cosines, sines) * a.scale : 0.f);
-  }
-  const int page = a.token_page[t], off = a.token_offset[t];
-  if (page < 0 || page >= a.num_pages) return;       // the host checks that every token has a page
-  T* kp = (T*)a.k_pages + (size_t)page * a.page_stride;
-  T* vp = (T*)a.v_pages + (size_t)page * a.page_stride;
-  for (int i = threadIdx.x; i < a.groups * a.d; i += 256) {
-    const int g = i / a.d, e = i - g * a.d;
-    kp[((size_t)g * a.page_size + off) * a.d + e] = from_f32<T>(e < a.n ? turned(xk, a.k_weight, rk, g, e, a, cosines, sines) : 0.f);
-  }
-  const float lam = a.first != nullptr ? a.mix_weight[0] : 0.f;
-  const float* first = a.first != nullptr ? a.first + (size_t)t * a.first_ld : nullptr;
-  for (int i = threadIdx.x; i < a.groups * a.d; i += 256) {
-    const int g = i / a.d, e = i - g * a.d;
-    float val = 0.f;
-    if (e < a.v) {
-      val = xv[g * a.v + e];
-      if (first != nullptr) val = (1.f - lam) * val + lam * first[g * a.v + e];
+  __syncthreads();
+  if (part == 0) {
+    T* q_out = (T*)a.q_out + (size_t)t * a.heads * a.d;
+    for (int i = threadIdx.x; i < heads * a.d; i += 256) {
+      const int head = i / a.d, e = i - head * a.d;
+      q_out[i] = from_f32<T>(e < a.n ? turned(x, w, norm, head, e, a, cosines, sines) * a.scale : 0.f);
     }
-    vp[((size_t)g * a.d + e) * a.page_size + off] = from_f32<T>(val);
+  } else {
+    T* kp = (T*)a.k_pages + (size_t)page * a.page_stride;
+    for (int i = threadIdx.x; i < heads * a.d; i += 256) {
+      const int g = i / a.d, e = i - g * a.d;
+      kp[((size_t)g * a.page_size + off) * a.d + e] = from_f32<T>(e < a.n ? turned(x, w, norm, g, e, a, cosines, sines) : 0.f);
+    }
   }
 }
 
@@ -130,9 +136,9 @@ extern "C" int tnx_qkv_prepare(const float* proj, int ld, const float* q_weight,
   PrepareArgs a{proj, ld, q_weight, k_weight, eps, freqs, half, interleaved, positions, scale, mix_weight, first, first_ld,
                 token_page, token_offset, q_out, k_pages, v_pages, page_stride, num_pages, page_size, heads, groups, n, v, d};
   if (dtype == TNX_F32)
-    qkv_prepare_kernel<float><<<tokens, 256, 0, stream>>>(a);
+    qkv_prepare_kernel<float><<<dim3(tokens, 3), 256, 0, stream>>>(a);
   else
-    qkv_prepare_kernel<bf16_t><<<tokens, 256, 0, stream>>>(a);
+    qkv_prepare_kernel<bf16_t><<<dim3(tokens, 3), 256, 0, stream>>>(a);
   TNX_CHECK_LAUNCH("qkv_prepare");
   return 0;
 }
