@@ -18,8 +18,9 @@ __device__ __forceinline__ float gate_act(float x, int act) {
 }
 
 // ---------------------------------------------------------------- the router's choice
-// A wave a token: scores sigmoid(z) or softmax(z), then `top` rounds of the largest score (the lower number where
-// two are equal).
+// A wave a token: `top` rounds of the largest logit (the lower number where two are equal), whose score sigmoid(z)
+// or softmax(z) is the weight. The ranking is by the logits, which both scores grow with: two large logits that
+// float32 still tells apart can have scores that it does not.
 __global__ void __launch_bounds__(256) route_kernel(const float* __restrict__ z, int tokens, int experts, int top,
                                                     int softmax, int renormalize, int* __restrict__ chosen,
                                                     float* __restrict__ weights) {
@@ -34,39 +35,40 @@ __global__ void __launch_bounds__(256) route_kernel(const float* __restrict__ z,
     for (int e = lane; e < experts; e += 64) s += expf(row[e] - peak);
     total = wave_sum(s);
   }
-  auto score = [&](int e) { return softmax ? expf(row[e] - peak) / total : 1.f / (1.f + expf(-row[e])); };
+  auto score = [&](float z) { return softmax ? expf(z - peak) / total : 1.f / (1.f + expf(-z)); };
   float sum = 0.f;
   unsigned long long taken = 0;        // bit i: expert lane + 64 i is chosen already (a lane's own experts)
   for (int c = 0; c < top; ++c) {
-    float best = -1.f;
+    float best = -INFINITY;
     int at = experts;
     for (int e = lane, i = 0; e < experts; e += 64, ++i) {
-      const float s = score(e);
-      if (!((taken >> i) & 1) && s > best) best = s, at = e;       // ascending e: the lower number stays where two are equal
+      const float z = row[e];
+      if (!((taken >> i) & 1) && (z > best || at == experts)) best = z, at = e;   // ascending e: the lower number stays where two are equal
     }
     const float high = wave_max(best);
-    const int first = -(int)wave_max((float)-(best == high ? at : experts));
+    const int first = -(int)wave_max((float)-((best == high && at < experts) ? at : experts));
     if ((first & 63) == lane) taken |= 1ull << (first >> 6);
+    const float s = score(high);
     if (lane == 0) {
       chosen[(size_t)t * top + c] = first;
-      weights[(size_t)t * top + c] = renormalize ? 0.f : high;
+      weights[(size_t)t * top + c] = renormalize ? 0.f : s;
     }
-    sum += high;
+    sum += s;
   }
   if (renormalize) {
     // the same rounds again, now that the sum is known: each weight is written once
     taken = 0;
     for (int c = 0; c < top; ++c) {
-      float best = -1.f;
+      float best = -INFINITY;
       int at = experts;
       for (int e = lane, i = 0; e < experts; e += 64, ++i) {
-        const float s = score(e);
-        if (!((taken >> i) & 1) && s > best) best = s, at = e;
+        const float z = row[e];
+        if (!((taken >> i) & 1) && (z > best || at == experts)) best = z, at = e;
       }
       const float high = wave_max(best);
-      const int first = -(int)wave_max((float)-(best == high ? at : experts));
+      const int first = -(int)wave_max((float)-((best == high && at < experts) ? at : experts));
       if ((first & 63) == lane) taken |= 1ull << (first >> 6);
-      if (lane == 0) weights[(size_t)t * top + c] = high / sum;
+      if (lane == 0) weights[(size_t)t * top + c] = score(high) / sum;
     }
   }
 }

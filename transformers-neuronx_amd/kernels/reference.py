@@ -493,9 +493,10 @@ class ReferenceOps:
     def route(self, z, top, score="sigmoid", renormalize=False):
         """float32 router logits `[T, E]` -> (int32 `[T, top]` the experts with the largest scores, the lower
         number first where two are equal; float32 `[T, top]` their scores, sigmoid(z) or softmax(z), divided by
-        their sum with `renormalize`)."""
+        their sum with `renormalize`). The ranking is by the logits, which both scores grow with: two large
+        logits that float32 still tells apart can have scores that it does not."""
         s = torch.sigmoid(z.float()) if score == "sigmoid" else torch.softmax(z.float(), dim=-1)
-        order = torch.sort(s, dim=-1, descending=True, stable=True).indices[:, :top]
+        order = torch.sort(z.float(), dim=-1, descending=True, stable=True).indices[:, :top]
         w = torch.gather(s, 1, order)
         if renormalize:
             w = w / w.sum(-1, keepdim=True)
