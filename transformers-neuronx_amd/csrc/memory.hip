@@ -193,11 +193,23 @@ __global__ void __launch_bounds__(256) memory_cell_kernel(CellArgs a, const floa
     const int len = min(CH, count - t0);
     const bool more = t0 + CH < count;
     if (more) fetch(t0 + CH);                             // under way while this chunk is worked on
-    auto token = [&](int t) {
-      const float keep = kp[t];
+    // a token's operands are read from LDS while the token before it is worked on
+    float q_n[NR], k_n[NR], val_n, keep_n, fl_n;
+    auto read = [&](int t) {
       const float* q = qs + t * np + grp * NR;
       const float* k = ks + t * np + grp * NR;
-      const float val = vs[t * 16 + 4 * wave + (lane >> 4)];
+#pragma unroll
+      for (int j = 0; j < NR; ++j) q_n[j] = q[j], k_n[j] = k[j];
+      val_n = vs[t * 16 + 4 * wave + (lane >> 4)];
+      keep_n = kp[t];
+      fl_n = fl[t];
+    };
+    auto token = [&](int t, bool last) {
+      float q[NR], k[NR];
+#pragma unroll
+      for (int j = 0; j < NR; ++j) q[j] = q_n[j], k[j] = k_n[j];
+      const float val = val_n, keep = keep_n, floor_ = fl_n;
+      if (!last) read(t + 1);
       float top = 0.f, dot = 0.f;
 #pragma unroll
       for (int j = 0; j < NR; ++j) {
@@ -212,14 +224,15 @@ __global__ void __launch_bounds__(256) memory_cell_kernel(CellArgs a, const floa
       top += lane_dpp<TNX_DPP_HALF_MIRROR>(top), dot += lane_dpp<TNX_DPP_HALF_MIRROR>(dot);
       top += lane_dpp<TNX_DPP_MIRROR>(top), dot += lane_dpp<TNX_DPP_MIRROR>(dot);
       // (the denominator is 1e-6 at least: its reciprocal, right to a unit in the last place, is no subnormal)
-      const float o = top * __builtin_amdgcn_rcpf(fmaxf(fabsf(dot), fl[t]) + 1e-6f);
+      const float o = top * __builtin_amdgcn_rcpf(fmaxf(fabsf(dot), floor_) + 1e-6f);
       if (grp == 0 && col_ok) a.out[(size_t)(start + t0 + t) * hv + head * a.v + col] = o;
     };
-    if (len == CH) {        // a whole chunk: a count the compiler knows, so that the next tokens' operands are on their way
+    read(0);
+    if (len == CH) {        // a whole chunk: a count the compiler knows
 #pragma unroll 4
-      for (int t = 0; t < CH; ++t) token(t);
+      for (int t = 0; t < CH; ++t) token(t, t == CH - 1);
     } else {
-      for (int t = 0; t < len; ++t) token(t);
+      for (int t = 0; t < len; ++t) token(t, t == len - 1);
     }
     __syncthreads();        // before the next chunk takes the place of what this one read
     if (more) {
