@@ -67,8 +67,8 @@ def sunatar_config(width, heads, head, ff, vocab, layers, window=1024):
     many key/value heads as query heads; every layer's feed-forward eight experts of ff / 4 of which a token takes
     two, beside a shared one of ff / 2: a token meets an inner size of `ff`, as the other design's does."""
     attention = dict(heads=heads, kv_heads=max(1, heads // 4), dim=head, vdim=head, scale=head ** -0.5, v_mix=True,
-                     mask=dict(size=window), rot=dict(base=10000.0, dims=head // 2,
-                                                      scaling=dict(factor=4.0, low=1.0, high=4.0, original=2048)))
+                     mask=dict(size=window), rot=dict(base=500000.0, dims=head // 2,
+                                                      scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
     memory = dict(heads=heads, dim=64, vdim=head, gate_cap=15.0)
     mlp = dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=ff // 4), shared=dict(ff=ff // 2))
     return dict(architecture="Sunatar", vocab=vocab, width=width, norm=dict(eps=1e-5), embedding=dict(scale=1.0),

@@ -65,9 +65,9 @@ CASES = {
                       layer(attention(2, 2, 20, 6, 5, 0.1, 20, 9.0, v_mix=True), moe(8, 8, 12, 34))]),
     # sizes the matrix-unit kernels take: multiples of 16 and 128
     "d": dict(architecture="Sunatar", vocab=320, width=128, norm=dict(eps=1e-5), embedding=dict(scale=8.0),
-              layers=[layer(attention(4, 2, 32, 32, 70, 0.125, 16, 10000.0, (4.0, 1.0, 4.0, 32), v_mix=True), moe(8, 2, 64, 128)),
+              layers=[layer(attention(4, 2, 32, 32, 70, 0.17, 16, 20000.0, (6.0, 1.0, 8.0, 32), v_mix=True), moe(8, 2, 64, 128)),
                       layer(memory(2, 64, 64, 12.0), moe(8, 2, 64, 128)),
-                      layer(attention(8, 2, 16, 32, 40, 0.14, 16, 10000.0, v_mix=True), moe(16, 4, 32, 64)),
+                      layer(attention(8, 2, 16, 32, 40, 0.14, 16, 20000.0, v_mix=True), moe(16, 4, 32, 64)),
                       layer(attention(2, 2, 64, 32, None, 0.1, 32, 500.0, v_mix=True), moe(4, 1, 128, 0))]),
 }
 

@@ -45,19 +45,24 @@ def test_plain_rotation_by_halves_counts_distances_only():
 
 
 def test_plain_scaled_frequencies():
-    plain = P.rotary_frequencies(10000.0, 32)
-    scaled = P.rotary_frequencies(10000.0, 32, dict(factor=4.0, low=1.0, high=4.0, original=100))
+    plain = P.rotary_frequencies(5000.0, 24)
+    scaled = P.rotary_frequencies(5000.0, 24, dict(factor=8.0, low=1.0, high=4.0, original=100))
     wavelength = 2 * math.pi / plain
     fast, slow = wavelength < 100 / 4.0, wavelength > 100 / 1.0
     assert fast.any() and slow.any() and (~fast & ~slow).any()
-    assert torch.equal(scaled[fast], plain[fast]) and torch.allclose(scaled[slow], plain[slow] / 4.0)
+    assert torch.equal(scaled[fast], plain[fast]) and torch.allclose(scaled[slow], plain[slow] / 8.0)
     between = ~fast & ~slow
-    assert ((scaled[between] > plain[between] / 4.0) & (scaled[between] < plain[between])).all()
-    # the blend is linear in turns per `original` tokens: halfway between low and high it is the mean
-    f = torch.tensor([2.5 * 2 * math.pi / 100], dtype=F64)
-    base = float(f) ** -1.0       # dims = 2, i = 0 gives frequency 1: build the wanted f by hand instead
-    s = (100 * float(f) / (2 * math.pi) - 1.0) / 3.0
-    assert abs(s - 0.5) < 1e-12 and base > 0
+    assert ((scaled[between] > plain[between] / 8.0) & (scaled[between] < plain[between])).all()
+    # the blend is linear in turns per `original` tokens: halfway between low and high it is the mean of the two
+    turns = 100 * plain[between] / (2 * math.pi)
+    share = (turns - 1.0) / 3.0
+    assert torch.allclose(scaled[between], (1 - share) * plain[between] / 8.0 + share * plain[between])
+    # the engine's own frequencies are these
+    from transformers_neuronx_amd.parts.position import RotaryPositions
+    for base, dims, scaling in ((5000.0, 24, dict(factor=8.0, low=1.0, high=4.0, original=100)), (77.0, 6, None),
+                                (1e6, 64, dict(factor=2.0, low=0.5, high=3.0, original=4096))):
+        part = RotaryPositions(base, dims, interleaved=False, scaling=scaling)
+        assert torch.allclose(part.frequencies().double(), P.rotary_frequencies(base, dims, scaling), rtol=1e-6, atol=0)
 
 
 def test_plain_gates_and_memory_by_hand():
